@@ -326,9 +326,11 @@ void moe_align(Tensor offsets, Tensor sorted, Tensor pos, Tensor ids, int64_t nu
 }  // namespace
 
 void register_seq_ops(pybind11::module& m);  // csrc/bindings_seq.cpp
+void register_lin_ops(pybind11::module& m);  // csrc/bindings_lin.cpp
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   register_seq_ops(m);
+  register_lin_ops(m);
   m.def("rms_norm_ext", &rms_norm_ext);
   m.def("post_norm_residual", &post_norm_residual);
   m.def("gated_act", &gated_act);

@@ -223,22 +223,30 @@ void gated_delta(Tensor out, Tensor qkv32, Tensor bg, Tensor gate, Tensor norm_w
 }
 
 // q [T, H * dim], k [T, G * dim], v [T, G * vdim]: column slices of ONE projection output
-void qkv_prep(Tensor q_out, Tensor cache, Tensor q, Tensor k, Tensor v, int64_t heads, int64_t kv_heads, int64_t dim,
-              int64_t vdim, OptTensor q_norm, OptTensor k_norm, int64_t rot_dims, OptTensor inv_freq, bool v_unit,
-              OptTensor v_lambda, OptTensor v_first, double eps, Tensor positions, Tensor slots) {
+void qkv_prep(Tensor q_out, Tensor cache, Tensor q, Tensor k, OptTensor v, int64_t heads, int64_t kv_heads,
+              int64_t dim, int64_t vdim, OptTensor q_norm, OptTensor k_norm, int64_t rot_dims, OptTensor inv_freq,
+              bool v_unit, OptTensor v_lambda, OptTensor v_first, double eps, Tensor positions, Tensor slots,
+              bool head_norm, double q_temp_coef, int64_t q_temp_every) {
   check_rows(q, "q");
   check_rows(k, "k");
-  check_rows(v, "v");
   die::QkvPrepArgs a;
   a.f32 = is_f32(q, "q");
   const int64_t T = q.size(0);
-  TORCH_CHECK(is_f32(k, "k") == a.f32 && is_f32(v, "v") == a.f32 && is_f32(q_out, "q_out") == a.f32 &&
-                  is_f32(cache, "cache") == a.f32,
+  TORCH_CHECK(is_f32(k, "k") == a.f32 && is_f32(q_out, "q_out") == a.f32 && is_f32(cache, "cache") == a.f32,
               "one dtype");
   TORCH_CHECK(heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0, "heads % kv_heads == 0");
-  TORCH_CHECK(q.size(1) == heads * dim && k.size(1) == kv_heads * dim && v.size(1) == kv_heads * vdim &&
-                  k.size(0) == T && v.size(0) == T && k.stride(0) == q.stride(0) && v.stride(0) == q.stride(0),
-              "q / k / v: slices of one projection");
+  TORCH_CHECK(q.size(1) == heads * dim && k.size(1) == kv_heads * dim && k.size(0) == T &&
+                  k.stride(0) == q.stride(0),
+              "q / k: slices of one projection");
+  if (v.has_value()) {
+    check_rows(*v, "v");
+    TORCH_CHECK(is_f32(*v, "v") == a.f32 && v->size(1) == kv_heads * vdim && v->size(0) == T &&
+                    v->stride(0) == q.stride(0),
+                "v: a slice of the same projection");
+  } else {
+    TORCH_CHECK(vdim == dim && !v_lambda.has_value(), "values taken from the keys: vdim == dim, no value mixing");
+  }
+  TORCH_CHECK(q_temp_coef == 0.0 || q_temp_every >= 1, "q_temp_every >= 1");
   TORCH_CHECK(q_out.is_contiguous() && q_out.numel() == T * heads * dim, "q_out [T, H * dim]");
   TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == kv_heads * (dim + vdim),
               "cache [blocks, block_size, G * (dim + vdim)]");
@@ -247,15 +255,19 @@ void qkv_prep(Tensor q_out, Tensor cache, Tensor q, Tensor k, Tensor v, int64_t 
   TORCH_CHECK(positions.numel() >= T && slots.numel() >= T, "positions, slots [T]");
   a.q = q.data_ptr();
   a.k = k.data_ptr();
-  a.v = v.data_ptr();
+  a.v = v.has_value() ? v->data_ptr() : nullptr;
   a.xstride = q.stride(0);
   a.T = (int)T;
   a.heads = (int)heads;
   a.kv_heads = (int)kv_heads;
   a.dim = (int)dim;
   a.vdim = (int)vdim;
-  a.q_norm = f32_ptr(q_norm, heads * dim, "q_norm");
-  a.k_norm = f32_ptr(k_norm, kv_heads * dim, "k_norm");
+  a.head_norm = head_norm;
+  TORCH_CHECK(!head_norm || q_norm.has_value(), "head_norm needs the norm weights");
+  a.q_norm = f32_ptr(q_norm, head_norm ? dim : heads * dim, "q_norm");
+  a.k_norm = f32_ptr(k_norm, head_norm ? dim : kv_heads * dim, "k_norm");
+  a.q_temp_coef = (float)q_temp_coef;
+  a.q_temp_every = (int)q_temp_every;
   a.rot_dims = (int)rot_dims;
   a.inv_freq = f32_ptr(inv_freq, rot_dims / 2, "inv_freq");
   a.v_unit = v_unit;
@@ -280,7 +292,8 @@ void qkv_prep(Tensor q_out, Tensor cache, Tensor q, Tensor k, Tensor v, int64_t 
 
 void sink_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables, OptTensor cu_q, Tensor ctx_lens,
                Tensor positions, OptTensor sink, OptTensor bias, int64_t max_q, int64_t heads, int64_t kv_heads,
-               int64_t dim, int64_t vdim, int64_t window, double scale, int64_t impl) {
+               int64_t dim, int64_t vdim, int64_t window, double scale, int64_t impl, double softcap,
+               OptTensor slopes) {
   die::SinkAttnArgs a;
   a.f32 = is_f32(q, "q");
   TORCH_CHECK(is_f32(out, "out") == a.f32 && is_f32(cache, "cache") == a.f32, "one dtype");
@@ -320,6 +333,9 @@ void sink_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables, OptTenso
     a.bias = bias->data_ptr<float>();
     a.bias_rows = (int)bias->size(0);
   }
+  TORCH_CHECK(softcap >= 0.0, "softcap >= 0");
+  a.softcap = (float)softcap;
+  a.slopes = f32_ptr(slopes, heads, "slopes");
   a.num_seqs = (int)S;
   a.total_q = (int)T;
   a.max_q = (int)max_q;

@@ -83,12 +83,15 @@ hipError_t launch_gated_delta(void* out, const float* qkv32, const float* bg, co
 struct QkvPrepArgs {
   const void* q;          // [T, H * dim], [T, G * dim], [T, G * vdim]: slices of one projection, row stride xstride
   const void* k;
-  const void* v;
+  const void* v;          // nullptr: the values are the keys as projected, before any norm or rotation (vdim == dim)
   int64_t xstride;
   bool f32;
   int T, heads, kv_heads, dim, vdim;
   const float* q_norm;    // [H * dim], [G * dim]: RMS norm over the whole projection, or nullptr
   const float* k_norm;
+  bool head_norm;         // q_norm and k_norm are [dim], shared by all heads: RMS norm of every head by itself
+  float q_temp_coef;      // != 0: q, after its norm, times 1 + coef * ln(floor((p + 1) / q_temp_every) + 1) at position p
+  int q_temp_every;
   int rot_dims;           // rotated dims per head (pairs i, i + rot_dims / 2), 0: none
   const float* inv_freq;  // [rot_dims / 2]
   bool v_unit;            // each value head divided by its root mean square
@@ -116,6 +119,8 @@ struct SinkAttnArgs {
   const float* sink;      // [H] or nullptr
   const float* bias;      // [bias_rows, H]: added to the scaled score of a key at distance n, row min(n, bias_rows - 1)
   int bias_rows;
+  float softcap;          // > 0: the scaled score s becomes softcap * tanh(s / softcap), before bias and slope
+  const float* slopes;    // [H] or nullptr: slopes[h] * n is taken off the score of a key at distance n
   int num_seqs, total_q, max_q, heads, kv_heads, dim, vdim, block_size;
   int window;             // keys j with 0 <= p - j < window (0: all j <= p)
   float scale;

@@ -577,6 +577,7 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
   float lam = 0.f;
   if (a.v_lambda != nullptr) lam = a.v_lambda[0];
   // bf16 with head sizes that are multiples of 8: 16-byte loads and stores, 8 values per thread and trip
+  const bool v_is_k = a.v == nullptr;   // values = keys as projected
   const bool wide = !f32 && d % 8 == 0 && dv % 8 == 0 && a.xstride % 8 == 0 && aligned16(a.q) && aligned16(a.k) &&
                     aligned16(a.v) && aligned16(a.q_out) && aligned16(a.cache) &&
                     (a.v_first == nullptr || (a.vfstride % 8 == 0 && aligned16(a.v_first)));
@@ -584,7 +585,7 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
     const bf16_t* qp = reinterpret_cast<const bf16_t*>(a.q) + t * a.xstride;
     const bf16_t* kp = reinterpret_cast<const bf16_t*>(a.k) + t * a.xstride;
     const bf16_t* vp = reinterpret_cast<const bf16_t*>(a.v) + t * a.xstride;
-    for (int c8 = threadIdx.x; c8 < (nq + nk + nv) / 8; c8 += NT) {
+    for (int c8 = threadIdx.x; c8 < (v_is_k ? nq + nk : nq + nk + nv) / 8; c8 += NT) {
       const int c = 8 * c8;
       float f[8];
       if (c < nq) {
@@ -618,13 +619,29 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
       kv[c] = x;
       sk += x * x;
     }
-    for (int c = threadIdx.x; c < nv; c += NT) {
+    for (int c = threadIdx.x; c < (v_is_k ? 0 : nv); c += NT) {
       float x = ldv(a.v, t * a.xstride + c, f32);
       if (a.v_lambda != nullptr) x = (1.0f - lam) * x + lam * ldv(a.v_first, t * a.vfstride + c, f32);
       vv[c] = x;
     }
   }
-  if (a.q_norm != nullptr) {
+  if (v_is_k) {
+    __syncthreads();
+    for (int c = threadIdx.x; c < nk; c += NT) vv[c] = kv[c];
+  }
+  if (a.q_norm != nullptr && a.head_norm) {
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int hd = wave; hd < H + G; hd += NT / 64) {
+      float* base = hd < H ? qv + hd * d : kv + (hd - H) * d;
+      const float* w = hd < H ? a.q_norm : a.k_norm;
+      float ss = 0.f;
+      for (int c = lane; c < d; c += 64) ss += base[c] * base[c];
+      ss = wave_sum(ss);
+      const float rs = 1.0f / sqrtf(ss / (float)d + a.eps);
+      for (int c = lane; c < d; c += 64) base[c] *= rs * w[c];
+    }
+  } else if (a.q_norm != nullptr) {
     sq = block_sum<NT>(sq, red);   // (a barrier: every thread's loads are in LDS)
     sk = block_sum<NT>(sk, red);
     const float rq = 1.0f / sqrtf(sq / (float)nq + a.eps), rk = 1.0f / sqrtf(sk / (float)nk + a.eps);
@@ -632,6 +649,12 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
     for (int c = threadIdx.x; c < nk; c += NT) kv[c] *= rk * a.k_norm[c];
   }
   __syncthreads();
+  if (a.q_temp_coef != 0.f) {
+    const int64_t p = a.positions[t];
+    const float qm = 1.0f + a.q_temp_coef * logf((float)((p + 1) / a.q_temp_every) + 1.0f);
+    for (int c = threadIdx.x; c < nq; c += NT) qv[c] *= qm;
+    __syncthreads();
+  }
   if (a.rot_dims > 0) {
     const int half = a.rot_dims / 2;
     const float p = (float)a.positions[t];
@@ -781,7 +804,9 @@ hipError_t launch_qkv_prep(const QkvPrepArgs& a, hipStream_t s) {
   if (a.T == 0) return hipSuccess;
   if (a.heads < 1 || a.kv_heads < 1 || a.heads % a.kv_heads != 0 || a.dim < 1 || a.vdim < 1 || a.rot_dims < 0 ||
       a.rot_dims > a.dim || (a.rot_dims & 1) || a.block_size < 1 || (a.rot_dims > 0 && a.inv_freq == nullptr) ||
-      ((a.q_norm == nullptr) != (a.k_norm == nullptr)) || (a.v_lambda != nullptr && a.v_first == nullptr))
+      ((a.q_norm == nullptr) != (a.k_norm == nullptr)) || (a.v_lambda != nullptr && a.v_first == nullptr) ||
+      (a.v == nullptr && (a.vdim != a.dim || a.v_lambda != nullptr)) || (a.head_norm && a.q_norm == nullptr) ||
+      (a.q_temp_coef != 0.f && a.q_temp_every < 1))
     return hipErrorInvalidValue;
   const size_t lds = sizeof(float) * ((size_t)a.heads * a.dim + (size_t)a.kv_heads * (a.dim + a.vdim));
   if (lds > 150 * 1024) return hipErrorInvalidValue;

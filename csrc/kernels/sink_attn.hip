@@ -33,6 +33,12 @@ template <bool F32> __device__ __forceinline__ void stt(void* p, int64_t i, floa
     reinterpret_cast<bf16_t*>(p)[i] = f2bf(v);
 }
 
+// tanh through one v_exp_f32 and one reciprocal: 1 - 2 / (2^(2 x log2 e) + 1); exact limits at +-inf
+__device__ __forceinline__ float fast_tanh(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * 2.885390081777927f);
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
 template <int BK, int CC, int RPW, bool F32>
 __global__ void __launch_bounds__(256) sink_attn_kernel(SinkAttnArgs a, int QS, int KS, int VS) {
   constexpr int RW = RPW * WAVES;
@@ -112,6 +118,8 @@ __global__ void __launch_bounds__(256) sink_attn_kernel(SinkAttnArgs a, int QS, 
       const int n = prow[i] - j;
       const bool valid = rok[i] && j <= jhi && n >= 0 && (a.window <= 0 || n < a.window);
       sc *= a.scale;
+      if (a.softcap > 0.f) sc = a.softcap * tanhf(sc / a.softcap);
+      if (valid && a.slopes != nullptr) sc -= a.slopes[hrow[i]] * (float)n;
       if (valid && a.bias != nullptr) sc += a.bias[(int64_t)min(n, a.bias_rows - 1) * H + hrow[i]];
       sc = valid ? sc : -INFINITY;
       const float mn = fmaxf(m[i], wave_max(sc));
@@ -276,6 +284,9 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
   const int prow = rok ? (int)a.positions[q0 + myrow / QPG] : -1;
   constexpr float LOG2E = 1.4426950408889634f;
   const float sl2 = a.scale * LOG2E;
+  const bool shaped = a.softcap > 0.f || a.slopes != nullptr;
+  const float capl2 = a.softcap * LOG2E, s_over_cap = a.softcap > 0.f ? a.scale / a.softcap : 0.f;
+  const float slope2 = a.slopes != nullptr ? a.slopes[myh] * LOG2E : 0.f;
   const bool has_sink = a.sink != nullptr && rok && z == 0;
   float m = has_sink ? a.sink[myh] * LOG2E : -1e30f;
   float l = has_sink ? 1.0f : 0.0f;
@@ -362,7 +373,21 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
     float mx = -INFINITY;
     const bool interior = wave_full && j0 + MKT - 1 <= min(pw_first, jhi) &&
                           (a.window <= 0 || pw_last - j0 < a.window);
-    if (interior) {
+    if (shaped) {
+      // capped scores and / or a linear distance penalty: cap * tanh(s * scale / cap) - slope * n, in log2 units
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int j = j0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
+        const int n = prow - j;
+        const bool valid = interior || (rok && j <= jhi && n >= 0 && (a.window <= 0 || n < a.window));
+        float v = a.softcap > 0.f ? capl2 * fast_tanh(sc[r] * s_over_cap) : sc[r] * sl2;
+        v -= slope2 * (float)n;
+        if (bias != nullptr && valid) v += bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
+        v = valid ? v : -INFINITY;
+        sc[r] = v;
+        mx = fmaxf(mx, v);
+      }
+    } else if (interior) {
       const bool far = bias == nullptr || prow - (j0 + 27 + 4 * hh) >= a.bias_rows - 1;
       if (far) {
 #pragma unroll
@@ -515,7 +540,7 @@ __global__ void __launch_bounds__(256) sink_attn_decode_kernel(SinkAttnArgs a, f
     float f[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (r < QPG && 8 * kl < D) unpack8(*reinterpret_cast<const uint4*>(qg + ((int64_t)s * H + g * QPG + r) * D + 8 * kl), f);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) qf[r][e] = f[e] * (a.scale * LOG2E);
+    for (int e = 0; e < 8; ++e) qf[r][e] = f[e] * (a.softcap > 0.f ? a.scale / a.softcap : a.scale * LOG2E);
   }
   if (tid < R) {
     const bool has_sink = a.sink != nullptr && tid < QPG && z == 0;
@@ -572,6 +597,8 @@ __global__ void __launch_bounds__(256) sink_attn_decode_kernel(SinkAttnArgs a, f
         if (kl == 0) {
           const int n = p - j;
           const bool valid = r < QPG && j <= jhi && n >= 0;
+          if (a.softcap > 0.f) d = a.softcap * LOG2E * fast_tanh(d);
+          if (valid && a.slopes != nullptr) d -= a.slopes[g * QPG + r] * LOG2E * (float)n;
           if (valid && a.bias != nullptr) d += a.bias[(int64_t)min(n, a.bias_rows - 1) * H + g * QPG + r] * LOG2E;
           sc[r * DCH + jj] = valid ? d : -INFINITY;
         }

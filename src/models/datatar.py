@@ -37,7 +37,7 @@ from typing import Any, Dict, List, Optional
 import torch
 import torch.nn.functional as F
 
-from src.ops import mix
+from src.ops import lin, mix
 from src.parallel.tp import TPContext
 
 
@@ -54,10 +54,16 @@ class LatentAttnSpec:
     window: int       # 0: every earlier position
     rot_base: float
     rot_dims: int     # rotated dims (pairs 2i, 2i + 1) at the start of the rotary part
+    has_sink: bool = True            # a per-head term exp(sink_h) in the softmax denominator
+    out_gate: bool = False           # head h's output times sigmoid(W_g a)_h, W_g [heads, hidden]
+    kv_from: Optional[int] = None    # no down-projection of its own: attends over that layer's cached latents
 
     @property
     def cache_width(self) -> int:
-        return self.kv_rank + self.rot_dim
+        return 0 if self.kv_from is not None else self.kv_rank + self.rot_dim
+
+    def state_shapes(self) -> Dict[str, Any]:
+        return {}
 
     @staticmethod
     def from_config(m: Dict[str, Any]) -> "LatentAttnSpec":
@@ -196,18 +202,24 @@ class LatentAttentionMixer:
             t = torch.empty(*shape, dtype=dtype, device=device)
             return t.normal_(0.0, scale, generator=gen) if gen is not None else t.zero_()
 
-        self.dqkv = rnd(s.q_rank + s.kv_rank + s.rot_dim, hidden)          # [W_dq; W_dkv]
+        # one input projection: [W_dq; W_dkv (unless the latents are another layer's); W_g (with an output gate)]
+        self.kvw = 0 if s.kv_from is not None else s.kv_rank + s.rot_dim
+        self.dqkv = rnd(s.q_rank + self.kvw + (s.heads if s.out_gate else 0), hidden)
         self.dq_norm = torch.ones(s.q_rank, dtype=dtype, device=device)
-        self.dkv_norm = torch.ones(s.kv_rank, dtype=dtype, device=device)
+        self.dkv_norm = torch.ones(s.kv_rank, dtype=dtype, device=device) if self.kvw else None
         self.uq = rnd(s.heads * (s.dim + s.rot_dim), s.q_rank, scale=std * 4)
         self.uk = rnd(s.heads, s.dim, s.kv_rank, scale=std * 4)            # W_uk, head by head: [H, dim, rank]
         self.uv_t = rnd(s.heads, s.kv_rank, s.vdim, scale=std * 4)         # W_uv^T head by head: [H, rank, vdim]
-        self.sink = torch.zeros(s.heads, dtype=torch.float32, device=device)
+        self.sink = torch.zeros(s.heads, dtype=torch.float32, device=device) if s.has_sink else None
         self.o = rnd(hidden, s.heads * s.vdim)
         self.inv_freq = mix.rope_inv_freq(s.rot_base, s.rot_dims, device)
 
+    def finalize(self) -> None:
+        """Nothing is derived from the weights."""
+
     def tensors(self) -> List[torch.Tensor]:
-        return [self.dqkv, self.dq_norm, self.dkv_norm, self.uq, self.uk, self.uv_t, self.sink, self.o]
+        return [t for t in (self.dqkv, self.dq_norm, self.dkv_norm, self.uq, self.uk, self.uv_t, self.sink, self.o)
+                if t is not None]
 
     def load(self, name: str, t: torch.Tensor) -> bool:
         """One checkpoint tensor ``<layer>.mix.<name>``; False if the name is not this mixer's."""
@@ -219,11 +231,13 @@ class LatentAttentionMixer:
 
         if name == "dq":
             return put(self.dqkv[: s.q_rank], t)
-        if name == "dkv":
-            return put(self.dqkv[s.q_rank:], t)
+        if name == "dkv" and self.kvw:
+            return put(self.dqkv[s.q_rank: s.q_rank + self.kvw], t)
+        if name == "g" and s.out_gate:
+            return put(self.dqkv[s.q_rank + self.kvw:], t)
         if name == "dq.norm":
             return put(self.dq_norm, t)
-        if name == "dkv.norm":
+        if name == "dkv.norm" and self.kvw:
             return put(self.dkv_norm, t)
         if name == "uq":
             return put(self.uq, t)
@@ -231,7 +245,7 @@ class LatentAttentionMixer:
             return put(self.uk, t.view(s.heads, s.dim, s.kv_rank))
         if name == "uv":
             return put(self.uv_t, t.view(s.heads, s.vdim, s.kv_rank).transpose(1, 2))
-        if name == "sink":
+        if name == "sink" and s.has_sink:
             return put(self.sink, t)
         if name == "o":
             return put(self.o, t)
@@ -239,22 +253,40 @@ class LatentAttentionMixer:
 
     def state(self) -> Dict[str, torch.Tensor]:
         s = self.spec
-        return {"dq": self.dqkv[: s.q_rank], "dkv": self.dqkv[s.q_rank:], "dq.norm": self.dq_norm,
-                "dkv.norm": self.dkv_norm, "uq": self.uq, "uk": self.uk.reshape(s.heads * s.dim, s.kv_rank),
-                "uv": self.uv_t.transpose(1, 2).reshape(s.heads * s.vdim, s.kv_rank), "sink": self.sink, "o": self.o}
+        out = {"dq": self.dqkv[: s.q_rank], "dq.norm": self.dq_norm, "uq": self.uq,
+               "uk": self.uk.reshape(s.heads * s.dim, s.kv_rank),
+               "uv": self.uv_t.transpose(1, 2).reshape(s.heads * s.vdim, s.kv_rank), "o": self.o}
+        if self.kvw:
+            out["dkv"], out["dkv.norm"] = self.dqkv[s.q_rank: s.q_rank + self.kvw], self.dkv_norm
+        if s.out_gate:
+            out["g"] = self.dqkv[s.q_rank + self.kvw:]
+        if s.has_sink:
+            out["sink"] = self.sink
+        return out
 
-    def forward(self, a: torch.Tensor, positions: torch.Tensor, meta, cache: torch.Tensor, eps: float) -> torch.Tensor:
+    def forward(self, a: torch.Tensor, positions: torch.Tensor, meta, cache: torch.Tensor, eps: float,
+                **_) -> torch.Tensor:
+        """``cache``: this layer's rows, or with ``kv_from`` the rows of the layer whose latents it shares (that
+        layer ran earlier in the step, so this step's tokens are already there)."""
         s = self.spec
         t = a.shape[0]
         p = mix.linear(a, self.dqkv)
-        cq = mix.latent_qkv_prep(p, s.q_rank, self.dq_norm, self.dkv_norm, cache, positions, meta.slot_mapping,
-                                 s.kv_rank, s.rot_dim, self.inv_freq, eps)
+        nq = s.q_rank
+        if self.kvw:
+            cq = mix.latent_qkv_prep(p[:, : nq + self.kvw], nq, self.dq_norm, self.dkv_norm, cache, positions,
+                                     meta.slot_mapping, s.kv_rank, s.rot_dim, self.inv_freq, eps)
+        else:
+            cq = mix.rms_norm_ext(p[:, :nq], self.dq_norm, eps)
         q = mix.linear(cq, self.uq)
         q_lat = torch.bmm(q.view(t, s.heads, s.dim + s.rot_dim)[:, :, : s.dim].transpose(0, 1), self.uk)
         o_lat = mix.latent_attn(q_lat, q, s.dim, cache, meta.block_tables, meta.cu_q if meta.is_prefill else None,
                                 meta.ctx_lens, positions, self.sink, meta.max_q_len if meta.is_prefill else 1,
                                 s.window, s.scale, s.rot_dim, self.inv_freq)
-        o = torch.bmm(o_lat, self.uv_t).transpose(0, 1).reshape(t, s.heads * s.vdim)
+        o = torch.bmm(o_lat, self.uv_t)                                    # [H, T, vdim]
+        if s.out_gate:
+            o = lin.head_gate(o, p[:, nq + self.kvw:])
+        else:
+            o = o.transpose(0, 1).reshape(t, s.heads * s.vdim)
         return mix.linear(o, self.o)
 
 

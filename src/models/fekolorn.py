@@ -52,6 +52,13 @@ class SinkAttnSpec:
     v_unit: bool = False       # every value head divided by its root mean square
     v_mix: bool = False        # values blended with the first such layer's
     bias_max: float = 0.0      # > 0: learned bias per (distance bucket, head); the last bucket starts here
+    has_sink: bool = True      # a per-head term exp(sink_h) in the softmax denominator
+    head_norm: bool = False    # with qk_norm: every head normed by itself, weights [dim] shared by the heads
+    v_from_k: bool = False     # no value projection: the values are the keys as projected, before their norm
+    softcap: float = 0.0       # > 0: scaled scores pass through softcap * tanh(s / softcap)
+    slope_exp: float = 0.0     # > 0: head h's score drops by 2^(-slope_exp (h + 1) / heads) per position of distance
+    q_temp_coef: float = 0.0   # != 0: q times 1 + coef * ln(floor((p + 1) / q_temp_every) + 1) at position p
+    q_temp_every: int = 1
 
     @property
     def cache_width(self) -> int:
@@ -243,13 +250,23 @@ class SinkAttentionMixer:
             t = torch.empty(*shape, dtype=dt, device=self.device)
             return t.normal_(0.0, scale, generator=gen) if gen is not None else t.zero_()
 
-        self.nq, self.nk, self.nv = s.heads * s.dim, s.kv_heads * s.dim, s.kv_heads * s.vdim
+        if s.v_from_k and (s.vdim != s.dim or s.v_mix):
+            raise ValueError("values taken from the keys: vdim must equal dim, and there is no value mixing")
+        if s.head_norm and not s.qk_norm:
+            raise ValueError("head_norm is a form of qk_norm")
+        self.nq, self.nk = s.heads * s.dim, s.kv_heads * s.dim
+        self.nv = 0 if s.v_from_k else s.kv_heads * s.vdim
         self.qkv = rnd(self.nq + self.nk + self.nv, hidden)
         self.o = rnd(hidden, s.heads * s.vdim)
         f32 = torch.float32
-        self.sink = rnd(s.heads, scale=0.5, dt=f32)
-        self.q_norm = (1.0 + rnd(self.nq, scale=0.1, dt=f32)) if s.qk_norm else None
-        self.k_norm = (1.0 + rnd(self.nk, scale=0.1, dt=f32)) if s.qk_norm else None
+        self.sink = rnd(s.heads, scale=0.5, dt=f32) if s.has_sink else None
+        self.q_norm = (1.0 + rnd(s.dim if s.head_norm else self.nq, scale=0.1, dt=f32)) if s.qk_norm else None
+        self.k_norm = (1.0 + rnd(s.dim if s.head_norm else self.nk, scale=0.1, dt=f32)) if s.qk_norm else None
+        # the distance penalty per head, rounded once from float64
+        self.slopes = None
+        if s.slope_exp:
+            hs = torch.arange(1, s.heads + 1, dtype=torch.float64)
+            self.slopes = torch.pow(2.0, -float(s.slope_exp) * hs / s.heads).float().to(self.device)
         self.vmix = (0.3 + rnd(1, scale=0.05, dt=f32)) if s.v_mix else None
         # buckets of the distance bias: a checkpoint's tensor decides (load); a random model takes up to 32, half
         # of them below bias_max
@@ -275,11 +292,11 @@ class SinkAttentionMixer:
             return _put(self.qkv[: self.nq], t)
         if name == "k":
             return _put(self.qkv[self.nq: self.nq + self.nk], t)
-        if name == "v":
+        if name == "v" and self.nv:
             return _put(self.qkv[self.nq + self.nk:], t)
         if name == "o":
             return _put(self.o, t)
-        if name == "sink":
+        if name == "sink" and self.sink is not None:
             return _put(self.sink, t)
         if name == "q.norm" and self.q_norm is not None:
             return _put(self.q_norm, t)
@@ -294,8 +311,11 @@ class SinkAttentionMixer:
         return False
 
     def state(self) -> Dict[str, torch.Tensor]:
-        out = {"q": self.qkv[: self.nq], "k": self.qkv[self.nq: self.nq + self.nk], "v": self.qkv[self.nq + self.nk:],
-               "o": self.o, "sink": self.sink}
+        out = {"q": self.qkv[: self.nq], "k": self.qkv[self.nq: self.nq + self.nk], "o": self.o}
+        if self.nv:
+            out["v"] = self.qkv[self.nq + self.nk:]
+        if self.sink is not None:
+            out["sink"] = self.sink
         if self.q_norm is not None:
             out["q.norm"], out["k.norm"] = self.q_norm, self.k_norm
         if self.vmix is not None:
@@ -308,7 +328,8 @@ class SinkAttentionMixer:
                shared: Dict[str, Any]) -> torch.Tensor:
         """p [T, >= nq + nk + nv]: this mixer's q | k | v columns of a projection output. Returns W_o attn."""
         s = self.spec
-        q, k, v = p[:, : self.nq], p[:, self.nq: self.nq + self.nk], p[:, self.nq + self.nk: self.nq + self.nk + self.nv]
+        q, k = p[:, : self.nq], p[:, self.nq: self.nq + self.nk]
+        v = p[:, self.nq + self.nk: self.nq + self.nk + self.nv] if self.nv else None
         v_first = lam = None
         if s.v_mix:
             if "v_first" in shared:
@@ -317,17 +338,18 @@ class SinkAttentionMixer:
                 shared["v_first"] = v   # a view: the projection output stays alive for the later layers
         qr = seq.qkv_prep(q, k, v, cache, s.heads, s.kv_heads, s.dim, s.vdim, positions, meta.slot_mapping, eps,
                           q_norm=self.q_norm, k_norm=self.k_norm, rot_dims=s.rot_dims, inv_freq=self.inv_freq,
-                          v_unit=s.v_unit, v_lambda=lam, v_first=v_first)
+                          v_unit=s.v_unit, v_lambda=lam, v_first=v_first, head_norm=s.head_norm,
+                          q_temp_coef=s.q_temp_coef, q_temp_every=s.q_temp_every)
         o = seq.sink_attn(qr, cache, meta.block_tables, meta.cu_q if meta.is_prefill else None, meta.ctx_lens,
                           positions, self.sink, self.bias, meta.max_q_len if meta.is_prefill else 1, s.heads,
-                          s.kv_heads, s.dim, s.vdim, s.window, s.scale)
+                          s.kv_heads, s.dim, s.vdim, s.window, s.scale, softcap=s.softcap, slopes=self.slopes)
         return mix.linear(o, self.o)
 
     def forward_streams(self, h, positions, meta, cache, eps, state, shared, rag):
         """(y1, y2, a1, a2): the mixer's output is a1 * y1 (+ a2 * y2)."""
         return self.attend(mix.linear(h, self.qkv), positions, meta, cache, eps, shared), None, 1.0, 1.0
 
-    def forward(self, a, positions, meta, cache, eps, state=None, shared=None):
+    def forward(self, a, positions, meta, cache, eps, state=None, shared=None, **_):
         return self.attend(mix.linear(a, self.qkv), positions, meta, cache, eps, shared if shared is not None else {})
 
 

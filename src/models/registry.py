@@ -4,7 +4,9 @@ Model-class registry: which model class serves a checkpoint directory, decided b
 * HuggingFace-format Llama / Mistral / Mixtral (``model_type``) -> :class:`src.models.llama.CausalLM`;
 * ``"architecture": "Datatar"`` (layers listed in the config) -> :class:`src.models.datatar.DatatarLM`;
 * ``"architecture": "Fekolorn"`` (layers listed in the config, per-sequence state) ->
-  :class:`src.models.fekolorn.FekolornLM`.
+  :class:`src.models.fekolorn.FekolornLM`;
+* ``"architecture": "Bapivik"`` (layers listed in the config, learned positions, depth-averaged layer results) ->
+  :class:`src.models.bapivik.BapivikLM`.
 
 A new family registers a (matcher, arch reader, model class) triple with :func:`register_family`.
 """
@@ -87,7 +89,20 @@ def _fekolorn_arch(path: str, **kw):
     return fekolorn_arch_from_dir(path, **kw)
 
 
+def _bapivik_cls():
+    from src.models.bapivik import BapivikLM
+
+    return BapivikLM
+
+
+def _bapivik_arch(path: str, **kw):
+    from src.models.bapivik import bapivik_arch_from_dir
+
+    return bapivik_arch_from_dir(path, **kw)
+
+
 register_family("datatar", lambda c: c.get("architecture") == "Datatar", _datatar_arch, _datatar_cls)
 register_family("fekolorn", lambda c: c.get("architecture") == "Fekolorn", _fekolorn_arch, _fekolorn_cls)
+register_family("bapivik", lambda c: c.get("architecture") == "Bapivik", _bapivik_arch, _bapivik_cls)
 register_family("llama", lambda c: "architecture" not in c and c.get("model_type", "llama") in
                 ("llama", "mistral", "mixtral"), _llama_arch, _llama_cls)

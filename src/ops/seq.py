@@ -251,28 +251,41 @@ class _HeadMajorView:
         self.v[slots // self.bs, :, slots % self.bs] = rows
 
 
-def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: torch.Tensor, heads: int, kv_heads: int,
-             dim: int, vdim: int, positions: torch.Tensor, slots: torch.Tensor, eps: float,
+def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], cache: torch.Tensor, heads: int,
+             kv_heads: int, dim: int, vdim: int, positions: torch.Tensor, slots: torch.Tensor, eps: float,
              q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None, rot_dims: int = 0,
              inv_freq: Optional[torch.Tensor] = None, v_unit: bool = False, v_lambda: Optional[torch.Tensor] = None,
-             v_first: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The step between the q/k/v projection and the attention, one launch: optional RMS norm of q and of k over the
-    whole projection (plain weights), optional rotate-half rotary on the first ``rot_dims`` dims of every head (pair
-    i, i + rot_dims / 2, angle position * inv_freq[i]), values either divided by their per-head root mean square or
-    blended as (1 - l) v + l v_first; writes the token's keys and values into the cache at slots[t] (< 0: skipped;
-    a block's interior is head-major, [G][block_size][k | v]) and returns q [T, H * dim]."""
+             v_first: Optional[torch.Tensor] = None, head_norm: bool = False, q_temp_coef: float = 0.0,
+             q_temp_every: int = 1) -> torch.Tensor:
+    """The step between the q/k/v projection and the attention, one launch: optional RMS norm of q and of k (plain
+    weights) over the whole projection or, with ``head_norm``, of every head by itself with weights [dim] shared by
+    the heads; optional query temperature, q times 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1) after its
+    norm; optional rotate-half rotary on the first ``rot_dims`` dims of every head (pair i, i + rot_dims / 2, angle
+    position * inv_freq[i]); values either divided by their per-head root mean square or blended as
+    (1 - l) v + l v_first; ``v`` None: the values are the keys as projected, before norm and rotation. Writes the
+    token's keys and values into the cache at slots[t] (< 0: skipped; a block's interior is head-major,
+    [G][block_size][k | v]) and returns q [T, H * dim]."""
     T = q.shape[0]
     if q.is_cuda:
         q_out = torch.empty(T, heads * dim, dtype=q.dtype, device=q.device)
         _kern().qkv_prep(q_out, cache, q, k, v, heads, kv_heads, dim, vdim, q_norm, k_norm, rot_dims, inv_freq, v_unit,
-                         v_lambda, v_first, eps, positions, slots)
+                         v_lambda, v_first, eps, positions, slots, head_norm, float(q_temp_coef), int(q_temp_every))
         return q_out
+    if v is None:
+        v = k
     qf, kf, vf = q.float(), k.float(), v.float()
     if v_lambda is not None:
         vf = (1.0 - v_lambda) * vf + v_lambda * v_first.float()
-    if q_norm is not None:
+    if q_norm is not None and head_norm:
+        qh, kh = qf.view(T, heads, dim), kf.view(T, kv_heads, dim)
+        qf = (qh / torch.sqrt((qh * qh).mean(-1, keepdim=True) + eps) * q_norm).reshape(T, heads * dim)
+        kf = (kh / torch.sqrt((kh * kh).mean(-1, keepdim=True) + eps) * k_norm).reshape(T, kv_heads * dim)
+    elif q_norm is not None:
         qf = qf / torch.sqrt((qf * qf).mean(-1, keepdim=True) + eps) * q_norm
         kf = kf / torch.sqrt((kf * kf).mean(-1, keepdim=True) + eps) * k_norm
+    if q_temp_coef:
+        steps = torch.div(positions + 1, q_temp_every, rounding_mode="floor").float()
+        qf = qf * (1.0 + q_temp_coef * torch.log(steps + 1.0))[:, None]
     if rot_dims:
         half = rot_dims // 2
         ang = positions.float()[:, None] * inv_freq[None, :]
@@ -298,16 +311,18 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: torch.Ten
 def sink_attn(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, cu_q: Optional[torch.Tensor],
               ctx_lens: torch.Tensor, positions: torch.Tensor, sink: Optional[torch.Tensor],
               bias: Optional[torch.Tensor], max_q: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int,
-              scale: float, impl: int = 0) -> torch.Tensor:
+              scale: float, impl: int = 0, softcap: float = 0.0, slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Grouped-query attention over the cache that :func:`qkv_prep` writes. The query at position p sees the cached
-    positions j <= p with p - j < window (0: all); score (q . k_j) * scale + bias[min(p - j, rows - 1), h]; the
-    softmax denominator has one more term exp(sink[h]). Returns [T, H * vdim]. ``impl``: 0 = the matrix-core
-    kernel where it applies, 1 = the FMA kernel, 2 = the matrix-core kernel or an error."""
+    positions j <= p with p - j < window (0: all). Score: s = (q . k_j) * scale; with ``softcap`` > 0,
+    s <- softcap * tanh(s / softcap); then - slopes[h] * (p - j) (``slopes`` [H] fp32, a linear distance penalty)
+    and + bias[min(p - j, rows - 1), h]. The softmax denominator has one more term exp(sink[h]) when ``sink`` is
+    given. Returns [T, H * vdim]. ``impl``: 0 = the matrix-core kernel where it applies, 1 = the FMA kernel, 2 = the
+    matrix-core kernel or an error."""
     T = q.shape[0]
     if q.is_cuda:
         out = torch.empty(T, heads * vdim, dtype=q.dtype, device=q.device)
         _kern().sink_attn(out, q, cache, block_tables, cu_q, ctx_lens, positions, sink, bias, max_q, heads, kv_heads,
-                          dim, vdim, window, scale, impl)
+                          dim, vdim, window, scale, impl, float(softcap), slopes)
         return out
     bs = cache.shape[1]
     hm = _head_major(cache, kv_heads)
@@ -329,6 +344,10 @@ def sink_attn(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, 
             n = pos[t] - j
             ok = (n >= 0) & ((n < window) if window > 0 else torch.ones_like(n, dtype=torch.bool))
             sc = torch.einsum("hd,jhd->hj", qh[t], kk) * scale
+            if softcap:
+                sc = softcap * torch.tanh(sc / softcap)
+            if slopes is not None:
+                sc = sc - slopes[:, None] * n[None, :].float()
             if bias is not None:
                 sc = sc + bias[n.clamp(0, bias.shape[0] - 1)].T
             sc = sc.masked_fill(~ok[None, :], -math.inf)
