@@ -131,6 +131,10 @@ def parse(argv=None):
                    help="instead of the serving bench: Fekolorn beside the closest existing model (Llama) at equal "
                         "sizes, prefill / decode throughput and its kernels alone (bench/fekolorn_compare.py)")
     p.add_argument("--fekolorn-args", default="", help="arguments passed on to bench/fekolorn_compare.py")
+    p.add_argument("--bapivik-compare", action="store_true",
+                   help="instead of the serving benchmark: the Bapivik design beside Llama at equal "
+                        "sizes, prefill / decode throughput and its kernels alone (bench/bapivik_compare.py)")
+    p.add_argument("--bapivik-args", default="", help="arguments passed on to bench/bapivik_compare.py")
     return p.parse_args(argv)
 
 
@@ -479,6 +483,15 @@ def main(argv=None) -> int:
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
         return mod.main(shlex.split(args.fekolorn_args))
+    if args.bapivik_compare:  # likewise a separate measurement
+        import importlib.util
+        import shlex
+
+        spec = importlib.util.spec_from_file_location("bapivik_compare",
+                                                      os.path.join(ROOT, "bench", "bapivik_compare.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        return mod.main(shlex.split(args.bapivik_args))
     if needs_launcher(args):
         return self_launch(args, argv)
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -471,7 +471,7 @@ template <int NW> hipError_t launch_mfma_ndb(const LatentAttnArgs& a, hipStream_
   return hipErrorInvalidValue;
 }
 
-// Prompt-sized steps at the common rotary widths (rot_dim = 16 * NROT): the same algorithm with every wave's
+// Prompt-sized steps at the common rotary widths (rot_dim = 16 * NROT, NROT = 0: no rotary part): the same algorithm with every wave's
 // query fragments held in registers (loaded straight from global memory, the rotary part rotated on the way;
 // no query tile in LDS, so the per-tile LDS traffic is the key tile alone) and the key tile double-buffered
 // (one barrier per tile: the next tile's registers are stored into the other buffer after this tile's MFMAs).
@@ -711,15 +711,16 @@ template <int NDB, int NROT> hipError_t launch_mfma_rq(const LatentAttnArgs& a, 
   return hipGetLastError();
 }
 
-// the register-query kernel exists for rank in {64, 128, 256} x rot_dim in {16, 32, 64}; unsplit steps only
+// the register-query kernel exists for rank in {64, 128, 256} x rot_dim in {0, 16, 32, 64}; unsplit steps only
 inline bool mfma_rq_ok(const LatentAttnArgs& a) {
   const int r = a.sh.rank, t = a.sh.rot_dim;
   return a.nsplit <= 1 && (int64_t)a.max_q * a.heads > 32 && (r == 64 || r == 128 || r == 256) &&
-         (t == 16 || t == 32 || t == 64);
+         (t == 0 || t == 16 || t == 32 || t == 64);
 }
 
 template <int NDB> hipError_t launch_mfma_rq_rot(const LatentAttnArgs& a, hipStream_t s) {
   switch (a.sh.rot_dim) {
+    case 0: return launch_mfma_rq<NDB, 0>(a, s);   // no rotary part: latents without positions
     case 16: return launch_mfma_rq<NDB, 1>(a, s);
     case 32: return launch_mfma_rq<NDB, 2>(a, s);
     case 64: return launch_mfma_rq<NDB, 4>(a, s);

@@ -254,11 +254,22 @@ __global__ void __launch_bounds__(NT) bias_relu2_kernel(void* out, const void* z
 
 __global__ void __launch_bounds__(NT) head_gate_kernel(void* out, const void* o, const void* g, int64_t gstride,
                                                       bool f32, int T, int H, int v) {
+  extern __shared__ float gates[];   // [H]: the token's gates, one sigmoid per head
   const int64_t t = blockIdx.x;
+  for (int h = threadIdx.x; h < H; h += NT) gates[h] = sigmoidf(ldv(g, t * gstride + h, f32));
+  __syncthreads();
+  if (v % 4 == 0 && al16(out) && al16(o)) {
+    for (int e = 4 * threadIdx.x; e < H * v; e += 4 * NT) {
+      const int h = e / v, c = e - h * v;
+      const float gate = gates[h];
+      const float4 x = ld4(o, ((int64_t)h * T + t) * v + c, f32);
+      st4(out, t * H * v + e, f32, make_float4(x.x * gate, x.y * gate, x.z * gate, x.w * gate));
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < H * v; e += NT) {
     const int h = e / v, c = e % v;
-    const float gate = sigmoidf(ldv(g, t * gstride + h, f32));
-    stv(out, t * H * v + e, f32, ldv(o, ((int64_t)h * T + t) * v + c, f32) * gate);
+    stv(out, t * H * v + e, f32, ldv(o, ((int64_t)h * T + t) * v + c, f32) * gates[h]);
   }
 }
 
@@ -267,13 +278,27 @@ __global__ void __launch_bounds__(NT) norm_sigmoid_gate_kernel(void* out, const 
                                                               int n) {
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
+  const bool vec = n % 4 == 0 && gstride % 4 == 0 && al16(out) && al16(o) && al16(g) && al16(w);
   float ss = 0.f;
-  for (int c = threadIdx.x; c < n; c += NT) {
-    const float v = o[t * n + c];
-    ss += v * v;
+  if (vec) {
+    for (int c = 4 * threadIdx.x; c < n; c += 4 * NT) ss += sq4(f4(o, t * n + c));
+  } else {
+    for (int c = threadIdx.x; c < n; c += NT) {
+      const float x = o[t * n + c];
+      ss += x * x;
+    }
   }
   ss = block_sum<NT>(ss, red);
   const float rs = 1.0f / sqrtf(ss / (float)n + eps);
+  if (vec) {
+    for (int c = 4 * threadIdx.x; c < n; c += 4 * NT) {
+      const float4 x = f4(o, t * n + c), ww = f4(w, c), gg = ld4(g, t * gstride + c, f32);
+      st4(out, t * n + c, f32,
+          make_float4(x.x * rs * ww.x * sigmoidf(gg.x), x.y * rs * ww.y * sigmoidf(gg.y),
+                      x.z * rs * ww.z * sigmoidf(gg.z), x.w * rs * ww.w * sigmoidf(gg.w)));
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < n; c += NT)
     stv(out, t * n + c, f32, o[t * n + c] * rs * w[c] * sigmoidf(ldv(g, t * gstride + c, f32)));
 }
@@ -396,8 +421,9 @@ hipError_t launch_bias_relu2(void* out, const void* z, const void* b, bool f32, 
 hipError_t launch_head_gate(void* out, const void* o, const void* g, int64_t gstride, bool f32, int T, int H, int v,
                             hipStream_t s) {
   if (T == 0) return hipSuccess;
-  if (H <= 0 || v <= 0) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(head_gate_kernel, dim3(T), dim3(NT), 0, s, out, o, g, gstride, f32, T, H, v);
+  if (H <= 0 || H > 8192 || v <= 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(head_gate_kernel, dim3(T), dim3(NT), (size_t)H * sizeof(float), s, out, o, g, gstride, f32, T, H,
+                     v);
   return hipGetLastError();
 }
 

@@ -286,6 +286,7 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
   const float sl2 = a.scale * LOG2E;
   const bool shaped = a.softcap > 0.f || a.slopes != nullptr;
   const float capl2 = a.softcap * LOG2E, s_over_cap = a.softcap > 0.f ? a.scale / a.softcap : 0.f;
+  const float cap_m2 = -2.0f * capl2, s2_over_cap = s_over_cap * 2.885390081777927f;
   const float slope2 = a.slopes != nullptr ? a.slopes[myh] * LOG2E : 0.f;
   const bool has_sink = a.sink != nullptr && rok && z == 0;
   float m = has_sink ? a.sink[myh] * LOG2E : -1e30f;
@@ -374,18 +375,36 @@ __global__ void __launch_bounds__(64 * NW) sink_attn_mfma_kernel(SinkAttnArgs a,
     const bool interior = wave_full && j0 + MKT - 1 <= min(pw_first, jhi) &&
                           (a.window <= 0 || pw_last - j0 < a.window);
     if (shaped) {
-      // capped scores and / or a linear distance penalty: cap * tanh(s * scale / cap) - slope * n, in log2 units
+      // capped scores and / or a linear distance penalty: cap * tanh(s * scale / cap) - slope * n, in log2 units.
+      // tanh = 1 - 2 / (2^(2 x log2 e) + 1), so the capped score is one multiply-add of the reciprocal; the
+      // distance of score r is that of score 0 minus a constant
+      const float nf0 = (float)(prow - j0 - 4 * hh);
+      if (interior && bias == nullptr) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int j = j0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
-        const int n = prow - j;
-        const bool valid = interior || (rok && j <= jhi && n >= 0 && (a.window <= 0 || n < a.window));
-        float v = a.softcap > 0.f ? capl2 * fast_tanh(sc[r] * s_over_cap) : sc[r] * sl2;
-        v -= slope2 * (float)n;
-        if (bias != nullptr && valid) v += bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
-        v = valid ? v : -INFINITY;
-        sc[r] = v;
-        mx = fmaxf(mx, v);
+        for (int r = 0; r < 16; ++r) {
+          const float nf = nf0 - (float)((r & 3) + 8 * (r >> 2));
+          float v;
+          if (a.softcap > 0.f)
+            v = fmaf(cap_m2, __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(sc[r] * s2_over_cap) + 1.0f), capl2);
+          else
+            v = sc[r] * sl2;
+          v = fmaf(-slope2, nf, v);
+          sc[r] = v;
+          mx = fmaxf(mx, v);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int j = j0 + (r & 3) + 8 * (r >> 2) + 4 * hh;
+          const int n = prow - j;
+          const bool valid = interior || (rok && j <= jhi && n >= 0 && (a.window <= 0 || n < a.window));
+          float v = a.softcap > 0.f ? capl2 * fast_tanh(sc[r] * s_over_cap) : sc[r] * sl2;
+          v -= slope2 * (float)n;
+          if (bias != nullptr && valid) v += bias[(int64_t)min(n, a.bias_rows - 1) * H] * LOG2E;
+          v = valid ? v : -INFINITY;
+          sc[r] = v;
+          mx = fmaxf(mx, v);
+        }
       }
     } else if (interior) {
       const bool far = bias == nullptr || prow - (j0 + 27 + 4 * hh) >= a.bias_rows - 1;
