@@ -150,6 +150,13 @@ void bias_relu2(Tensor out, Tensor z, Tensor b) {
                                 cur_stream()));
 }
 
+void tanh_cap(Tensor out, Tensor z, double cap) {
+  const bool f = is_f32(z, "z");
+  check_c(out, at::kFloat, "out");
+  TORCH_CHECK(z.is_contiguous() && out.numel() == z.numel() && cap > 0.0, "tanh_cap: z contiguous, out fp32 of its size, cap > 0");
+  HIP_OK(die::launch_tanh_cap(out.data_ptr<float>(), z.data_ptr(), f, (float)cap, z.numel(), cur_stream()));
+}
+
 void head_gate(Tensor out, Tensor o, Tensor g) {
   const bool f = is_f32(o, "o");
   TORCH_CHECK(o.dim() == 3 && o.is_contiguous(), "o [H, T, v] contiguous");
@@ -227,6 +234,7 @@ void register_lin_ops(pybind11::module& m) {
   m.def("post_pre_norm", &post_pre_norm);
   m.def("depth_avg_norm", &depth_avg_norm);
   m.def("bias_relu2", &bias_relu2);
+  m.def("tanh_cap", &tanh_cap);
   m.def("head_gate", &head_gate);
   m.def("norm_sigmoid_gate", &norm_sigmoid_gate);
   m.def("lightning_attn", &lightning_attn);

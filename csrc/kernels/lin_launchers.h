@@ -61,6 +61,9 @@ hipError_t launch_depth_avg_norm(const DepthAvgArgs& a, hipStream_t s);
 // out[r, c] = relu(z[r, c] + b[c])^2
 hipError_t launch_bias_relu2(void* out, const void* z, const void* b, bool f32, int rows, int n, hipStream_t s);
 
+// out[i] (fp32) = cap * tanh(z[i] / cap), cap > 0
+hipError_t launch_tanh_cap(float* out, const void* z, bool f32, float cap, int64_t total, hipStream_t s);
+
 // out[t, h * v + c] = o[h, t, c] * sigmoid(g[t * gstride + h]): per-head output gate, fused with the move from
 // head-major to token-major
 hipError_t launch_head_gate(void* out, const void* o, const void* g, int64_t gstride, bool f32, int T, int H, int v,

@@ -8,6 +8,7 @@
 //   depth_avg_norm       the layer's last post-norm, the weighted average over all layer results so far and the
 //                        next layer's first norm (or the final norm), one launch
 //   bias_relu2           relu(z + b)^2
+//   tanh_cap             cap * tanh(z / cap) into fp32 (capped logits)
 //   head_gate            per-head sigmoid gate fused with the head-major -> token-major move
 //   norm_sigmoid_gate    rms(o) * w * sigmoid(g)
 //   lightning_attn       S <- decay S + k v^T, o = S^T q: one workgroup per (sequence, head), the state in
@@ -252,6 +253,13 @@ __global__ void __launch_bounds__(NT) bias_relu2_kernel(void* out, const void* z
   }
 }
 
+__global__ void __launch_bounds__(NT) tanh_cap_kernel(float* out, const void* z, bool f32, float cap, int64_t total) {
+  const int64_t stride = (int64_t)gridDim.x * NT;
+  const float inv = 1.0f / cap;
+  for (int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x; i < total; i += stride)
+    out[i] = cap * tanhf(ldv(z, i, f32) * inv);
+}
+
 __global__ void __launch_bounds__(NT) head_gate_kernel(void* out, const void* o, const void* g, int64_t gstride,
                                                       bool f32, int T, int H, int v) {
   extern __shared__ float gates[];   // [H]: the token's gates, one sigmoid per head
@@ -415,6 +423,15 @@ hipError_t launch_bias_relu2(void* out, const void* z, const void* b, bool f32, 
   const int64_t blocks = (total + 4 * NT - 1) / (4 * NT);
   hipLaunchKernelGGL(bias_relu2_kernel, dim3((unsigned)(blocks < 8192 ? blocks : 8192)), dim3(NT), 0, s, out, z, b,
                      f32, n, total);
+  return hipGetLastError();
+}
+
+hipError_t launch_tanh_cap(float* out, const void* z, bool f32, float cap, int64_t total, hipStream_t s) {
+  if (total == 0) return hipSuccess;
+  if (!(cap > 0.f)) return hipErrorInvalidValue;
+  const int64_t blocks = (total + NT - 1) / NT;
+  hipLaunchKernelGGL(tanh_cap_kernel, dim3((unsigned)(blocks < 8192 ? blocks : 8192)), dim3(NT), 0, s, out, z, f32,
+                     cap, total);
   return hipGetLastError();
 }
 

@@ -463,6 +463,6 @@ class BapivikLM:
         """fp32 logits [rows, vocab] = cap * tanh(embed . hidden / cap) (no cap: the products themselves)."""
         if argmax_parts is not None:
             raise ValueError("this head writes no per-tile argmax candidates")
-        z = mix.linear(hidden, self.embed).float()
+        z = mix.linear(hidden, self.embed)
         cap = self.arch.logit_softcap
-        return torch.tanh(z / cap) * cap if cap else z
+        return lin.tanh_cap(z, cap) if cap else z.float()

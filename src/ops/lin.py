@@ -7,7 +7,7 @@ Ops for layer stacks with sandwich norms and depth-weighted averaging, and for d
   in one launch (a norm after one sublayer and before the next);
 * :func:`depth_avg_norm` — a layer's last post-norm, the learned weighted average over the results of all layers so
   far, and the next layer's first norm (or the model's final norm) in one launch;
-* :func:`bias_relu2` — ``relu(z + b)^2``;
+* :func:`bias_relu2` — ``relu(z + b)^2``; :func:`tanh_cap` — ``cap * tanh(z / cap)`` into fp32 (capped logits);
 * :func:`head_gate`, :func:`norm_sigmoid_gate` — sigmoid output gates, one per head or one per channel after an RMS
   norm over all heads;
 * :func:`lightning_attn` — linear attention with a fixed decay per head and an fp32 matrix state per (sequence,
@@ -86,6 +86,16 @@ def bias_relu2(z: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         return out
     x = torch.relu((z.float() + b.float()).to(z.dtype).float())
     return (x * x).to(z.dtype)
+
+
+def tanh_cap(z: torch.Tensor, cap: float) -> torch.Tensor:
+    """cap * tanh(z / cap) as fp32, any shape."""
+    if z.is_cuda:
+        z = z.contiguous()
+        out = torch.empty(z.shape, dtype=torch.float32, device=z.device)
+        _kern().tanh_cap(out, z, float(cap))
+        return out
+    return torch.tanh(z.float() / cap) * cap
 
 
 def head_gate(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:

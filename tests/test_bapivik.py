@@ -225,6 +225,10 @@ def test_activation_and_gates(device):
             z, b = torch.randn(7, n, generator=g).to(dt), torch.randn(n, generator=g).to(dt)
             got = lin.bias_relu2(z.to(device), b.to(device)).cpu().double()
             assert torch.allclose(got, torch.relu(z.to(F64) + b.to(F64)) ** 2, atol=tol, rtol=tol)
+        z = (torch.randn(5, 19, generator=g) * 20).to(dt)
+        got = lin.tanh_cap(z.to(device), 7.5).cpu()
+        assert got.dtype == torch.float32
+        assert torch.allclose(got.double(), 7.5 * torch.tanh(z.to(F64) / 7.5), atol=1e-5, rtol=1e-5)
         H, T, v = 3, 6, 5
         o = torch.randn(H, T, v, generator=g).to(dt)
         gt = torch.randn(T, H + 4, generator=g).to(dt)
