@@ -625,21 +625,36 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
       vv[c] = x;
     }
   }
-  if (v_is_k) {
+  const bool per_head = a.q_norm != nullptr && a.head_norm;
+  float qm = 1.0f;   // query temperature
+  if (a.q_temp_coef != 0.f) {
+    const int64_t p = a.positions[t];
+    qm = 1.0f + a.q_temp_coef * logf((float)((p + 1) / a.q_temp_every) + 1.0f);
+  }
+  if (v_is_k && !per_head) {
     __syncthreads();
     for (int c = threadIdx.x; c < nk; c += NT) vv[c] = kv[c];
   }
-  if (a.q_norm != nullptr && a.head_norm) {
+  if (per_head) {
+    // 16 lanes per head, 16 heads at a time: sum of squares, then one pass that also keeps the raw key as the value
+    // (values taken from the keys) and folds the query temperature into the q heads' factor
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int hd = wave; hd < H + G; hd += NT / 64) {
+    const int grp = threadIdx.x >> 4, gl = threadIdx.x & 15;
+    for (int hd = grp; hd < H + G; hd += NT / 16) {
       float* base = hd < H ? qv + hd * d : kv + (hd - H) * d;
       const float* w = hd < H ? a.q_norm : a.k_norm;
+      float* raw = (v_is_k && hd >= H) ? vv + (hd - H) * d : nullptr;
       float ss = 0.f;
-      for (int c = lane; c < d; c += 64) ss += base[c] * base[c];
-      ss = wave_sum(ss);
-      const float rs = 1.0f / sqrtf(ss / (float)d + a.eps);
-      for (int c = lane; c < d; c += 64) base[c] *= rs * w[c];
+      for (int c = gl; c < d; c += 16) ss += base[c] * base[c];
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      float rs = 1.0f / sqrtf(ss / (float)d + a.eps);
+      if (hd < H) rs *= qm;
+      for (int c = gl; c < d; c += 16) {
+        const float x = base[c];
+        if (raw != nullptr) raw[c] = x;
+        base[c] = x * rs * w[c];
+      }
     }
   } else if (a.q_norm != nullptr) {
     sq = block_sum<NT>(sq, red);   // (a barrier: every thread's loads are in LDS)
@@ -649,9 +664,7 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
     for (int c = threadIdx.x; c < nk; c += NT) kv[c] *= rk * a.k_norm[c];
   }
   __syncthreads();
-  if (a.q_temp_coef != 0.f) {
-    const int64_t p = a.positions[t];
-    const float qm = 1.0f + a.q_temp_coef * logf((float)((p + 1) / a.q_temp_every) + 1.0f);
+  if (a.q_temp_coef != 0.f && !per_head) {
     for (int c = threadIdx.x; c < nq; c += NT) qv[c] *= qm;
     __syncthreads();
   }
