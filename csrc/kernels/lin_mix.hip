@@ -234,22 +234,29 @@ __global__ void __launch_bounds__(NT) depth_avg_norm_kernel(DepthAvgArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------- elementwise
-__global__ void __launch_bounds__(NT) bias_relu2_kernel(void* out, const void* z, const void* b, bool f32, int n,
-                                                       int64_t total) {
-  const bool vec = n % 4 == 0 && al16(out) && al16(z) && al16(b);
-  const int64_t stride = (int64_t)gridDim.x * NT;
-  if (vec) {
-    for (int64_t i = ((int64_t)blockIdx.x * NT + threadIdx.x) * 4; i < total; i += 4 * stride) {
-      const float4 v = ld4(z, i, f32), bb = ld4(b, i % n, f32);
-      const float x0 = fmaxf(rnd(v.x + bb.x, f32), 0.f), x1 = fmaxf(rnd(v.y + bb.y, f32), 0.f),
-                  x2 = fmaxf(rnd(v.z + bb.z, f32), 0.f), x3 = fmaxf(rnd(v.w + bb.w, f32), 0.f);
-      st4(out, i, f32, make_float4(x0 * x0, x1 * x1, x2 * x2, x3 * x3));
+// grid (column tiles, rows): no division per element; bf16 rows of a multiple of 8 columns move 16 bytes per access
+__global__ void __launch_bounds__(NT) bias_relu2_kernel(void* out, const void* z, const void* b, bool f32, int n) {
+  const int64_t r0 = (int64_t)blockIdx.y * n;
+  if (!f32 && n % 8 == 0 && al16(out) && al16(z) && al16(b)) {
+    const int c = 8 * (blockIdx.x * NT + threadIdx.x);
+    if (c >= n) return;
+    float v[8], bb[8];
+    unpack8(*reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(z) + r0 + c), v);
+    unpack8(*reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(b) + c), bb);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float x = fmaxf(rnd(v[e] + bb[e], false), 0.f);
+      v[e] = x * x;
     }
+    *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(out) + r0 + c) = pack8(v);
     return;
   }
-  for (int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x; i < total; i += stride) {
-    const float x = fmaxf(rnd(ldv(z, i, f32) + ldv(b, i % n, f32), f32), 0.f);
-    stv(out, i, f32, x * x);
+  for (int e = 0; e < 8; ++e) {
+    const int c = 8 * blockIdx.x * NT + e * NT + threadIdx.x;
+    if (c < n) {
+      const float x = fmaxf(rnd(ldv(z, r0 + c, f32) + ldv(b, c, f32), f32), 0.f);
+      stv(out, r0 + c, f32, x * x);
+    }
   }
 }
 
@@ -419,10 +426,13 @@ hipError_t launch_depth_avg_norm(const DepthAvgArgs& a, hipStream_t s) {
 hipError_t launch_bias_relu2(void* out, const void* z, const void* b, bool f32, int rows, int n, hipStream_t s) {
   if (rows == 0) return hipSuccess;
   if (n <= 0) return hipErrorInvalidValue;
-  const int64_t total = (int64_t)rows * n;
-  const int64_t blocks = (total + 4 * NT - 1) / (4 * NT);
-  hipLaunchKernelGGL(bias_relu2_kernel, dim3((unsigned)(blocks < 8192 ? blocks : 8192)), dim3(NT), 0, s, out, z, b,
-                     f32, n, total);
+  // rows ride in grid.y (at most 65535 per launch)
+  for (int r = 0; r < rows; r += 65535) {
+    const int nr = rows - r < 65535 ? rows - r : 65535;
+    const size_t off = (size_t)r * n * (f32 ? 4 : 2);
+    hipLaunchKernelGGL(bias_relu2_kernel, dim3((unsigned)((n + 8 * NT - 1) / (8 * NT)), (unsigned)nr), dim3(NT), 0, s,
+                       static_cast<char*>(out) + off, static_cast<const char*>(z) + off, b, f32, n);
+  }
   return hipGetLastError();
 }
 
