@@ -383,6 +383,82 @@ def test_attention_other_shapes(device):
             assert float((got - want).abs().max()) < 2e-5 * float(want.abs().max())
 
 
+def _latent_case(device, dt, n_ctx, q_lo, standout, present=True, block=16):
+    """Two mixers of the engine: A caches its latents for n_ctx tokens; B (``kv_from``) runs the queries
+    q_lo .. n_ctx - 1 over A's scattered pages. The input of token ``standout`` is chosen so that its latent lines up
+    with head 0's last query in latent space (score about 16, every other one about N(0, 3)). Returns (B's output,
+    the oracle's) for the query rows."""
+    from src.models.bapivik import BAPIVIK_MIXERS
+    from src.models.llama import AttnMetadata
+
+    g = torch.Generator().manual_seed(n_ctx + 3 * standout)
+    Wd, eps = 40, 1e-5
+    la = orc.latent_layer(heads=2, dim=16, vdim=16, kv_rank=32, q_rank=24, ff=0)
+    lb = orc.latent_layer(heads=3, dim=16, vdim=24, kv_rank=32, q_rank=16, kv_from=0, ff=0)
+    config = orc.make_config([la, lb], width=Wd)
+    w = {k: v.to(F64) for k, v in orc.random_weights(config, 4, dtype=dt).items()}
+    wa = {k[7:]: v for k, v in w.items() if k.startswith("l0.mix.")}
+    wb = {k[7:]: v for k, v in w.items() if k.startswith("l1.mix.")}
+    ha = torch.randn(n_ctx, Wd, generator=g).to(dt).to(F64)
+    hb = torch.randn(n_ctx, Wd, generator=g).to(dt).to(F64)
+    mb = dict(lb["mixer"])
+    # head 0's last query in latent space, and an input whose latent points that way
+    q_last = (orc.rms(hb[-1:] @ wb["dq"].T, wb["dq.norm"], eps) @ wb["uq"].T)[0, :16]
+    u = wb["uk"][:16].T @ q_last                                     # [kv_rank]
+    if present:
+        ha[standout] = (torch.linalg.pinv(wa["dkv"]) @ (u / wa["dkv.norm"])).to(dt).to(F64)
+    c = orc.latent(ha, wa, eps)
+    mb["scale"] = 16.0 / float(c[standout].norm() * u.norm()) if present else 16.0 / float(math.sqrt(32) * u.norm())
+    want = orc.latent_attention(hb, c, wb, mb, eps)[q_lo:]
+    # the engine's mixers on their own cache tensor
+    spec_a, spec_b = BAPIVIK_MIXERS["latent_attention"][1](la["mixer"]), BAPIVIK_MIXERS["latent_attention"][1](mb)
+    A = BAPIVIK_MIXERS["latent_attention"][0](spec_a, Wd, device, dt, None, 0.0)
+    B = BAPIVIK_MIXERS["latent_attention"][0](spec_b, Wd, device, dt, None, 0.0)
+    for mixer, ww in ((A, wa), (B, wb)):
+        for name, t in ww.items():
+            assert mixer.load(name, t.float()), name
+    nb = (n_ctx + block - 1) // block
+    perm = torch.randperm(nb + 2, generator=g)[:nb]
+    cache = torch.zeros(nb + 2, block, 32, dtype=dt, device=device)
+    pos = torch.arange(n_ctx)
+    slots = (perm[pos // block] * block + pos % block).to(device)
+    bt = perm[None].to(torch.int32).to(device)
+    ctx = torch.tensor([n_ctx], dtype=torch.int32, device=device)
+
+    def meta(lo):
+        n = n_ctx - lo
+        if n == 1:
+            return AttnMetadata(is_prefill=False, slot_mapping=slots[lo:], block_tables=bt, ctx_lens=ctx)
+        return AttnMetadata(is_prefill=True, slot_mapping=slots[lo:], block_tables=bt, ctx_lens=ctx,
+                            cu_q=torch.tensor([0, n], dtype=torch.int32, device=device), max_q_len=n)
+
+    A.forward(ha.to(dt).to(device), pos.to(device), meta(0), cache, eps)
+    assert B.spec.cache_width == 0 and B.dkv_norm is None
+    got = B.forward(hb[q_lo:].to(dt).to(device), pos[q_lo:].to(device), meta(q_lo), cache, eps)
+    return got.cpu().double(), want
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("where", ["far", "page", "first"])
+@pytest.mark.parametrize("rows", ["portion", "decode"])
+def test_latent_attention_on_shared_latents_far_keys(device, where, rows):
+    """A layer without latents of its own finds a key far back among 300, on a page border and at position 0 in the
+    pages another layer wrote — in a prompt portion and for a single decode row; fp32 (FMA kernel) and, on the GPU,
+    bf16 (matrix cores)."""
+    _need(device)
+    n_ctx = 300
+    standout = {"far": 2, "page": 255, "first": 0}[where]
+    q_lo = n_ctx - 1 if rows == "decode" else n_ctx - 45
+    for dt in ((torch.float32,) if device == "cpu" else (torch.float32, torch.bfloat16)):
+        got, want = _latent_case(device, dt, n_ctx, q_lo, standout)
+        tol = 3e-5 if dt == torch.float32 else 4e-2
+        assert float((got - want).abs().max()) < tol * float(want.abs().max())
+        _, without = _latent_case(device, dt, n_ctx, q_lo, standout, present=False)
+        # the engine's last row is much nearer to the oracle with that key than to the oracle without it
+        near, away = float((got[-1] - want[-1]).abs().max()), float((got[-1] - without[-1]).abs().max())
+        assert near < 0.15 * away, (near, away)
+
+
 # -------------------------------------------------------------------------------------------------- whole models
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("name", sorted(CONFIGS))
