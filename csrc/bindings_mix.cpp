@@ -52,7 +52,7 @@ void rms_norm_ext(Tensor out, Tensor x, OptTensor w, bool unit_offset, double ep
                                   unit_offset, (float)eps, (int)x.size(0), (int)x.size(1), cur_stream()));
 }
 
-void post_norm_residual(Tensor resid, OptTensor act, Tensor y, Tensor w, bool unit_offset, double eps) {
+void post_norm_residual(Tensor resid, OptTensor act, Tensor y, Tensor w, bool unit_offset, double eps, double mult) {
   TORCH_CHECK(resid.is_cuda() && resid.scalar_type() == at::kFloat && resid.is_contiguous() && resid.dim() == 2,
               "resid must be a contiguous fp32 [rows, n] GPU tensor");
   check_rows(y, "y");
@@ -68,7 +68,7 @@ void post_norm_residual(Tensor resid, OptTensor act, Tensor y, Tensor w, bool un
     ap = act->data_ptr();
   }
   HIP_OK(die::launch_post_norm_residual(resid.data_ptr<float>(), ap, y.data_ptr(), y.stride(0), yf, w.data_ptr(), wf,
-                                        unit_offset, (float)eps, (int)resid.size(0), (int)resid.size(1),
+                                        unit_offset, (float)eps, (float)mult, (int)resid.size(0), (int)resid.size(1),
                                         cur_stream()));
 }
 
@@ -105,11 +105,15 @@ void topk_sigmoid(Tensor w, Tensor ids, Tensor z) {
                                   (int)z.size(1), (int)w.size(1), cur_stream()));
 }
 
-void gather_scaled(Tensor xs, Tensor x, OptTensor sorted, Tensor w, int64_t topk) {
+void gather_scaled(Tensor xs, Tensor x, OptTensor sorted, OptTensor w, int64_t topk) {
   const bool f = is_f32(x, "x");
-  check_i(w, at::kFloat, "w");
+  const float* wp = nullptr;
+  if (w.has_value()) {
+    check_i(*w, at::kFloat, "w");
+    wp = w->data_ptr<float>();
+  }
   TORCH_CHECK(is_f32(xs, "xs") == f && xs.is_contiguous() && x.is_contiguous() && xs.dim() == 2 && x.dim() == 2 &&
-                  xs.size(1) == x.size(1) && xs.size(0) == x.size(0) * topk && w.numel() == xs.size(0),
+                  xs.size(1) == x.size(1) && xs.size(0) == x.size(0) * topk && (!w.has_value() || w->numel() == xs.size(0)),
               "gather_scaled shapes");
   const int* sp = nullptr;
   if (sorted.has_value()) {
@@ -117,8 +121,101 @@ void gather_scaled(Tensor xs, Tensor x, OptTensor sorted, Tensor w, int64_t topk
     TORCH_CHECK(sorted->numel() == xs.size(0), "sorted [T * K]");
     sp = sorted->data_ptr<int>();
   }
-  HIP_OK(die::launch_gather_scaled(xs.data_ptr(), x.data_ptr(), f, sp, w.data_ptr<float>(), (int)xs.size(0),
+  HIP_OK(die::launch_gather_scaled(xs.data_ptr(), x.data_ptr(), f, sp, wp, (int)xs.size(0),
                                    (int)topk, (int)x.size(1), cur_stream()));
+}
+
+const float* opt_f32(const OptTensor& t, int64_t n, const char* name) {
+  if (!t.has_value()) return nullptr;
+  check_i(*t, at::kFloat, name);
+  TORCH_CHECK(t->numel() == n, name, ": expected ", n, " values");
+  return t->data_ptr<float>();
+}
+
+void route_softmax_topk(Tensor w, Tensor ids, OptTensor gate, Tensor x, Tensor wr, int64_t n_route, OptTensor corr) {
+  check_rows(x, "x");
+  const bool xf = is_f32(x, "x"), wf = is_f32(wr, "wr");
+  check_i(w, at::kFloat, "w");
+  check_i(ids, at::kInt, "ids");
+  const int64_t T = x.size(0);
+  TORCH_CHECK(wr.dim() == 2 && wr.is_contiguous() && wr.size(1) == x.size(1) &&
+                  wr.size(0) >= n_route + (gate.has_value() ? 1 : 0),
+              "wr [>= n_route (+ 1 with a gate), H]");
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == T && ids.sizes() == w.sizes() && w.size(1) <= n_route,
+              "w, ids [T, K], K <= n_route");
+  float* gp = const_cast<float*>(opt_f32(gate, T, "gate"));
+  HIP_OK(die::launch_route_softmax_topk(w.data_ptr<float>(), ids.data_ptr<int>(), gp, x.data_ptr(), x.stride(0), xf,
+                                        wr.data_ptr(), wf, opt_f32(corr, n_route, "corr"), (int)T, (int)x.size(1),
+                                        (int)n_route, (int)w.size(1), cur_stream()));
+}
+
+void topk_softmax_corrected(Tensor w, Tensor ids, OptTensor gate, Tensor z, int64_t n_route, OptTensor corr) {
+  check_i(w, at::kFloat, "w");
+  check_i(ids, at::kInt, "ids");
+  check_i(z, at::kFloat, "z");
+  TORCH_CHECK(z.dim() == 2 && w.dim() == 2 && w.size(0) == z.size(0) && ids.sizes() == w.sizes() &&
+                  w.size(1) <= n_route && z.size(1) >= n_route + (gate.has_value() ? 1 : 0),
+              "z [T, >= n_route (+ 1 with a gate)]; w, ids [T, K], K <= n_route");
+  float* gp = const_cast<float*>(opt_f32(gate, z.size(0), "gate"));
+  HIP_OK(die::launch_topk_softmax_corrected(w.data_ptr<float>(), ids.data_ptr<int>(), gp, z.data_ptr<float>(),
+                                            (int)z.size(1), opt_f32(corr, n_route, "corr"), (int)z.size(0),
+                                            (int)n_route, (int)w.size(1), cur_stream()));
+}
+
+void combine_weighted(OptTensor out, OptTensor resid, OptTensor act, Tensor ys, OptTensor pos, Tensor x, Tensor wk,
+                      Tensor ids, int64_t num_experts, OptTensor extra, OptTensor gate, OptTensor w, bool unit_offset,
+                      double eps, double mult) {
+  const bool f = is_f32(x, "x");
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous(), "x [T, H] contiguous");
+  const int64_t T = x.size(0), H = x.size(1);
+  check_i(wk, at::kFloat, "wk");
+  check_i(ids, at::kInt, "ids");
+  TORCH_CHECK(wk.dim() == 2 && wk.size(0) == T && ids.sizes() == wk.sizes(), "wk, ids [T, K]");
+  const int64_t K = wk.size(1);
+  TORCH_CHECK(is_f32(ys, "ys") == f && ys.is_contiguous() && ys.dim() == 2 && ys.size(1) == H &&
+                  (ys.size(0) == T * K || num_experts == 0),
+              "ys [T * K, H] in x's dtype");
+  const int* pp = nullptr;
+  if (pos.has_value()) {
+    check_i(*pos, at::kInt, "pos");
+    TORCH_CHECK(pos->numel() == T * K, "pos [T * K]");
+    pp = pos->data_ptr<int>();
+  }
+  const void* ep = nullptr;
+  if (extra.has_value()) {
+    TORCH_CHECK(is_f32(*extra, "extra") == f && extra->is_contiguous() && extra->dim() == 2 && extra->size(0) == T &&
+                    extra->size(1) == H,
+                "extra [T, H] in x's dtype");
+    ep = extra->data_ptr();
+  }
+  TORCH_CHECK(!gate.has_value() || extra.has_value(), "gate without extra");
+  float* op = nullptr;
+  if (out.has_value()) {
+    check_i(*out, at::kFloat, "out");
+    TORCH_CHECK(out->dim() == 2 && out->size(0) == T && out->size(1) == H, "out [T, H]");
+    op = out->data_ptr<float>();
+  }
+  float* rp = nullptr;
+  void* ap = nullptr;
+  const void* wp = nullptr;
+  bool wf = false;
+  if (resid.has_value()) {
+    check_i(*resid, at::kFloat, "resid");
+    TORCH_CHECK(resid->dim() == 2 && resid->size(0) == T && resid->size(1) == H && w.has_value(), "resid [T, H], with w");
+    rp = resid->data_ptr<float>();
+    wf = is_f32(*w, "w");
+    TORCH_CHECK(w->is_contiguous() && w->numel() == H, "w [H]");
+    wp = w->data_ptr();
+    if (act.has_value()) {
+      TORCH_CHECK(is_f32(*act, "act") == f && act->is_contiguous() && act->sizes() == resid->sizes(),
+                  "act: x's dtype, the residual's shape");
+      ap = act->data_ptr();
+    }
+  }
+  TORCH_CHECK(op != nullptr || rp != nullptr, "out or resid");
+  HIP_OK(die::launch_combine_weighted(op, rp, ap, ys.data_ptr(), f, pp, x.data_ptr(), wk.data_ptr<float>(),
+                                      ids.data_ptr<int>(), (int)num_experts, ep, opt_f32(gate, T, "gate"), (int)T,
+                                      (int)K, (int)H, wp, wf, unit_offset, (float)eps, (float)mult, cur_stream()));
 }
 
 void combine_sum(Tensor out, Tensor ys, OptTensor pos, OptTensor extra, int64_t topk) {
@@ -327,10 +424,15 @@ void moe_align(Tensor offsets, Tensor sorted, Tensor pos, Tensor ids, int64_t nu
 
 void register_seq_ops(pybind11::module& m);  // csrc/bindings_seq.cpp
 void register_lin_ops(pybind11::module& m);  // csrc/bindings_lin.cpp
+void register_rec_ops(pybind11::module& m);  // csrc/bindings_rec.cpp
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   register_seq_ops(m);
   register_lin_ops(m);
+  register_rec_ops(m);
+  m.def("route_softmax_topk", &route_softmax_topk);
+  m.def("topk_softmax_corrected", &topk_softmax_corrected);
+  m.def("combine_weighted", &combine_weighted);
   m.def("rms_norm_ext", &rms_norm_ext);
   m.def("post_norm_residual", &post_norm_residual);
   m.def("gated_act", &gated_act);

@@ -226,7 +226,7 @@ void gated_delta(Tensor out, Tensor qkv32, Tensor bg, Tensor gate, Tensor norm_w
 void qkv_prep(Tensor q_out, Tensor cache, Tensor q, Tensor k, OptTensor v, int64_t heads, int64_t kv_heads,
               int64_t dim, int64_t vdim, OptTensor q_norm, OptTensor k_norm, int64_t rot_dims, OptTensor inv_freq,
               bool v_unit, OptTensor v_lambda, OptTensor v_first, double eps, Tensor positions, Tensor slots,
-              bool head_norm, double q_temp_coef, int64_t q_temp_every) {
+              bool head_norm, double q_temp_coef, int64_t q_temp_every, bool norm_after_rot) {
   check_rows(q, "q");
   check_rows(k, "k");
   die::QkvPrepArgs a;
@@ -263,6 +263,9 @@ void qkv_prep(Tensor q_out, Tensor cache, Tensor q, Tensor k, OptTensor v, int64
   a.dim = (int)dim;
   a.vdim = (int)vdim;
   a.head_norm = head_norm;
+  TORCH_CHECK(!norm_after_rot || (head_norm && v.has_value()),
+              "norm_after_rot is a form of head_norm, and not for values taken from the keys");
+  a.norm_after_rot = norm_after_rot;
   TORCH_CHECK(!head_norm || q_norm.has_value(), "head_norm needs the norm weights");
   a.q_norm = f32_ptr(q_norm, head_norm ? dim : heads * dim, "q_norm");
   a.k_norm = f32_ptr(k_norm, head_norm ? dim : kv_heads * dim, "k_norm");

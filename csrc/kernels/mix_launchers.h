@@ -14,12 +14,12 @@ namespace die {
 hipError_t launch_rms_norm_ext(void* out, int64_t ostride, bool out_f32, const void* x, int64_t xstride, bool in_f32,
                                const void* w, bool w_f32, bool unit_offset, float eps, int rows, int n,
                                hipStream_t s);
-// resid[r] (fp32) += y[r] / sqrt(mean(y[r]^2) + eps) * (w or 1 + w); act[r] (optional, bf16) = resid[r]
+// resid[r] (fp32) += mult * y[r] / sqrt(mean(y[r]^2) + eps) * (w or 1 + w); act[r] (optional, bf16) = resid[r]
 hipError_t launch_post_norm_residual(float* resid, void* act, const void* y, int64_t ystride, bool y_f32,
-                                     const void* w, bool w_f32, bool unit_offset, float eps, int rows, int n,
-                                     hipStream_t s);
+                                     const void* w, bool w_f32, bool unit_offset, float eps, float mult, int rows,
+                                     int n, hipStream_t s);
 // out[r, :f] = act(gu[r, :f]) * f(gu[r, f:2f]).  kind 0: silu(g) * u.  kind 1: g' = min(g, limit),
-// u' = clamp(u, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1)
+// u' = clamp(u, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1).  kind 2: gelu(g) * u, tanh form
 hipError_t launch_gated_act(void* out, const void* gu, bool f32, int rows, int f, int kind, float limit, float alpha,
                             hipStream_t s);
 
@@ -29,7 +29,23 @@ hipError_t launch_route_sigmoid_topk(float* w, int* ids, const void* x, int64_t 
                                      bool wr_f32, int T, int H, int E, int K, hipStream_t s);
 // the same selection from fp32 logits z [T, E] computed elsewhere
 hipError_t launch_topk_sigmoid(float* w, int* ids, const float* z, int T, int E, int K, hipStream_t s);
-// xs[j] = w[sorted[j]] * x[sorted[j] / K]  (sorted == nullptr: j itself)
+// Router with softmax scores over E choices: z = x . Wr[e] in fp32, s = softmax(z); the K largest s + corr (corr
+// optional; lowest index on ties) are chosen; w [T, K] = their s over the sum of the chosen s (+ 1e-20).
+// gate != nullptr: Wr has one more row, gate[t] = sigmoid(x . Wr[E]).
+hipError_t launch_route_softmax_topk(float* w, int* ids, float* gate, const void* x, int64_t xstride, bool x_f32,
+                                     const void* wr, bool wr_f32, const float* corr, int T, int H, int E, int K,
+                                     hipStream_t s);
+// the same selection from fp32 logits z [T, zstride] computed elsewhere (the gate's logit at column E)
+hipError_t launch_topk_softmax_corrected(float* w, int* ids, float* gate, const float* z, int zstride,
+                                         const float* corr, int T, int E, int K, hipStream_t s);
+// sum[t] = sum_k wk[t, k] * (ids[t, k] < E ? ys[pos[t * K + k]] : x[t]) + gate[t] * extra[t]  (pos == nullptr:
+// t * K + k; extra, gate optional). out != nullptr: out[t] (fp32) = sum[t]. resid != nullptr:
+// resid[t] += mult * rmsnorm(sum[t]) * (w or 1 + w), act[t] (optional, the activation type) = resid[t].
+hipError_t launch_combine_weighted(float* out, float* resid, void* act, const void* ys, bool f32, const int* pos,
+                                   const void* x, const float* wk, const int* ids, int E, const void* extra,
+                                   const float* gate, int T, int K, int H, const void* w, bool w_f32, bool unit_offset,
+                                   float eps, float mult, hipStream_t s);
+// xs[j] = w[sorted[j]] * x[sorted[j] / K]  (sorted == nullptr: j itself; w == nullptr: a plain gather)
 hipError_t launch_gather_scaled(void* xs, const void* x, bool f32, const int* sorted, const float* w, int n, int K,
                                 int H, hipStream_t s);
 // out[t] (fp32) = sum_k ys[pos[t * K + k]] (+ extra[t]);  pos == nullptr: t * K + k

@@ -55,7 +55,7 @@ __device__ __forceinline__ bool aligned16(const void* p) { return (reinterpret_c
 
 __global__ void __launch_bounds__(NT) post_norm_residual_kernel(float* resid, void* act, const void* y,
                                                                int64_t ystride, bool y_f32, const void* w, bool w_f32,
-                                                               bool unit, float eps, int n) {
+                                                               bool unit, float eps, float mult, int n) {
   __shared__ float red[NT / 64];
   const int64_t r = blockIdx.x;
   // bf16 rows of a multiple of 8 columns: 16-byte loads and stores, 8 columns per thread and trip
@@ -70,7 +70,7 @@ __global__ void __launch_bounds__(NT) post_norm_residual_kernel(float* resid, vo
       for (int q = 0; q < 8; ++q) ss += f[q] * f[q];
     }
     ss = block_sum<NT>(ss, red);
-    const float rs = 1.0f / sqrtf(ss / (float)n + eps);
+    const float rs = mult / sqrtf(ss / (float)n + eps);
     float4* rr = reinterpret_cast<float4*>(resid + r * n);
     for (int c = threadIdx.x; c < n / 8; c += NT) {
       float f[8], g[8];
@@ -86,7 +86,7 @@ __global__ void __launch_bounds__(NT) post_norm_residual_kernel(float* resid, vo
     }
     return;
   }
-  const float rs = row_rs(y, r * ystride, y_f32, n, eps, red);
+  const float rs = mult * row_rs(y, r * ystride, y_f32, n, eps, red);
   for (int c = threadIdx.x; c < n; c += NT) {
     float g = w ? ldv(w, c, w_f32) : 1.0f;
     if (unit) g += 1.0f;
@@ -98,6 +98,7 @@ __global__ void __launch_bounds__(NT) post_norm_residual_kernel(float* resid, vo
 
 __device__ __forceinline__ float gate1(float g, float u, int kind, float limit, float alpha) {
   if (kind == 0) return g / (1.0f + expf(-g)) * u;
+  if (kind == 2) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
@@ -204,7 +205,7 @@ __global__ void __launch_bounds__(NT) gather_scaled_kernel(void* xs, const void*
   const int64_t j = blockIdx.x;
   const int flat = sorted ? sorted[j] : (int)j;
   const int64_t t = flat / K;
-  const float wk = w[flat];
+  const float wk = w ? w[flat] : 1.0f;
   if (!f32 && H % 8 == 0 && aligned16(x) && aligned16(xs)) {
     const uint4* xp = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(x) + t * H);
     uint4* op = reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(xs) + j * H);
@@ -248,6 +249,161 @@ __global__ void __launch_bounds__(NT) combine_sum_kernel(float* out, const void*
       a += ldv(ys, j * H + c, f32);
     }
     out[t * H + c] = a;
+  }
+}
+
+// Softmax-scored selection of one token from its logits z[0 .. E): the K largest softmax(z) + corr (lowest index on
+// ties); weights = the chosen scores without corr, over their sum + 1e-20. `sc` [E] is scratch (LDS or registers'
+// spill), left holding the scores.
+__device__ __forceinline__ void softmax_select(const float* z, float* sc, const float* corr, int E, int K, float* w_out,
+                                               int* id_out) {
+  float mx = -INFINITY;
+  for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
+  float den = 0.f;
+  for (int e = 0; e < E; ++e) {
+    sc[e] = expf(z[e] - mx);
+    den += sc[e];
+  }
+  const float inv = 1.0f / den;
+  for (int e = 0; e < E; ++e) sc[e] *= inv;
+  uint64_t taken[ROUTE_E_MAX / 64] = {0, 0, 0, 0};
+  float sum = 0.f;
+  for (int k = 0; k < K; ++k) {
+    int bi = -1;
+    float bv = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float v = sc[e] + (corr ? corr[e] : 0.f);
+      if (v != v || ((taken[e >> 6] >> (e & 63)) & 1ull)) continue;
+      if (bi < 0 || v > bv) {
+        bv = v;
+        bi = e;
+      }
+    }
+    if (bi < 0) bi = 0;
+    taken[bi >> 6] |= 1ull << (bi & 63);
+    w_out[k] = sc[bi];
+    id_out[k] = bi;
+    sum += sc[bi];
+  }
+  const float rn = 1.0f / (sum + 1e-20f);
+  for (int k = 0; k < K; ++k) w_out[k] *= rn;
+}
+
+// One workgroup per token: wave v computes the logits of rows v, v + 4, ... of the router (E choices, then an
+// optional gate row); thread 0 selects.
+__global__ void __launch_bounds__(NT) route_softmax_topk_kernel(float* w_out, int* id_out, float* gate_out,
+                                                               const void* x, int64_t xstride, bool x_f32,
+                                                               const void* wr, bool wr_f32, const float* corr, int H,
+                                                               int E, int K) {
+  __shared__ float z[ROUTE_E_MAX + 1];
+  __shared__ float sc[ROUTE_E_MAX];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rows = E + (gate_out ? 1 : 0);
+  const bool vec = !x_f32 && !wr_f32 && H % 8 == 0 && xstride % 8 == 0 &&
+                   (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(wr) & 15) == 0;
+  for (int e = wave; e < rows; e += NT / 64) {
+    float a = 0.f;
+    if (vec) {
+      const uint4* xr = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(x) + (int64_t)t * xstride);
+      const uint4* wp = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(wr) + (int64_t)e * H);
+      for (int c = lane; c < H / 8; c += 64) {
+        float xf[8], wf[8];
+        unpack8(xr[c], xf);
+        unpack8(wp[c], wf);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) a += xf[q] * wf[q];
+      }
+    } else {
+      for (int c = lane; c < H; c += 64)
+        a += ldv(x, (int64_t)t * xstride + c, x_f32) * ldv(wr, (int64_t)e * H + c, wr_f32);
+    }
+    a = wave_sum(a);
+    if (lane == 0) z[e] = a;
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  softmax_select(z, sc, corr, E, K, w_out + (int64_t)t * K, id_out + (int64_t)t * K);
+  if (gate_out) gate_out[t] = 1.0f / (1.0f + expf(-z[E]));
+}
+
+// Selection alone, from logits already computed (a library fp32 GEMM for prompt-sized steps): one thread per token,
+// its scores in a slice of LDS.
+constexpr int SEL_NT = 64;
+__global__ void __launch_bounds__(SEL_NT) topk_softmax_corrected_kernel(float* w_out, int* id_out, float* gate_out,
+                                                                       const float* z, int zstride, const float* corr,
+                                                                       int T, int E, int K) {
+  extern __shared__ float scs[];   // [SEL_NT][E]
+  const int t = blockIdx.x * SEL_NT + threadIdx.x;
+  if (t >= T) return;
+  const float* zr = z + (int64_t)t * zstride;
+  softmax_select(zr, scs + threadIdx.x * E, corr, E, K, w_out + (int64_t)t * K, id_out + (int64_t)t * K);
+  if (gate_out) gate_out[t] = 1.0f / (1.0f + expf(-zr[E]));
+}
+
+// The weighted sum of a token's experts: sum_k wk[t, k] * (ids[t, k] < E ? ys[pos[t, k]] : x[t]) + gate[t] * extra[t]
+// (an id >= E names an identity expert, whose output is the token's input). out != nullptr: the sum as fp32.
+// resid != nullptr: resid[t] += mult * rmsnorm(sum) * (w | 1 + w) and act[t] (optional, the activation type) =
+// resid[t]; the sum is staged in LDS between its statistics and the update.
+__global__ void __launch_bounds__(NT) combine_weighted_kernel(float* out, float* resid, void* act, const void* ys,
+                                                             bool f32, const int* pos, const void* x, const float* wk,
+                                                             const int* ids, int E, const void* extra,
+                                                             const float* gate, int K, int H, const void* w, bool w_f32,
+                                                             bool unit, float eps, float mult) {
+  extern __shared__ float acc[];   // [H]
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const float gt = extra ? (gate ? gate[t] : 1.0f) : 0.f;
+  float ss = 0.f;
+  const bool vec = !f32 && H % 8 == 0 && aligned16(ys) && aligned16(x) && (extra == nullptr || aligned16(extra));
+  if (vec) {
+    for (int c = threadIdx.x; c < H / 8; c += NT) {
+      float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (extra) {
+        unpack8(reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(extra) + t * H)[c], a);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) a[q] *= gt;
+      }
+      for (int k = 0; k < K; ++k) {
+        const float wt = wk[t * K + k];
+        const bool ident = ids[t * K + k] >= E;
+        const int64_t j = pos ? pos[t * K + k] : t * K + k;
+        const bf16_t* src = ident ? reinterpret_cast<const bf16_t*>(x) + t * H : reinterpret_cast<const bf16_t*>(ys) + j * H;
+        float v[8];
+        unpack8(reinterpret_cast<const uint4*>(src)[c], v);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) a[q] += wt * v[q];
+      }
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        acc[8 * c + q] = a[q];
+        ss += a[q] * a[q];
+      }
+    }
+  } else {
+    for (int c = threadIdx.x; c < H; c += NT) {
+      float a = extra ? gt * ldv(extra, t * H + c, f32) : 0.f;
+      for (int k = 0; k < K; ++k) {
+        const bool ident = ids[t * K + k] >= E;
+        const int64_t j = pos ? pos[t * K + k] : t * K + k;
+        a += wk[t * K + k] * (ident ? ldv(x, t * H + c, f32) : ldv(ys, j * H + c, f32));
+      }
+      acc[c] = a;
+      ss += a * a;
+    }
+  }
+  if (out != nullptr) {
+    __syncthreads();
+    for (int c = threadIdx.x; c < H; c += NT) out[t * H + c] = acc[c];
+  }
+  if (resid == nullptr) return;
+  ss = block_sum<NT>(ss, red);
+  const float rs = mult / sqrtf(ss / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += NT) {
+    float g = ldv(w, c, w_f32);
+    if (unit) g += 1.0f;
+    const float v = resid[t * H + c] + acc[c] * rs * g;
+    resid[t * H + c] = v;
+    if (act) stv(act, t * H + c, f32, v);
   }
 }
 
@@ -385,19 +541,19 @@ hipError_t launch_rms_norm_ext(void* out, int64_t ostride, bool out_f32, const v
 }
 
 hipError_t launch_post_norm_residual(float* resid, void* act, const void* y, int64_t ystride, bool y_f32,
-                                     const void* w, bool w_f32, bool unit_offset, float eps, int rows, int n,
-                                     hipStream_t s) {
+                                     const void* w, bool w_f32, bool unit_offset, float eps, float mult, int rows,
+                                     int n, hipStream_t s) {
   if (rows == 0) return hipSuccess;
   if (n <= 0) return hipErrorInvalidValue;
   hipLaunchKernelGGL(post_norm_residual_kernel, dim3(rows), dim3(NT), 0, s, resid, act, y, ystride, y_f32, w, w_f32,
-                     unit_offset, eps, n);
+                     unit_offset, eps, mult, n);
   return hipGetLastError();
 }
 
 hipError_t launch_gated_act(void* out, const void* gu, bool f32, int rows, int f, int kind, float limit, float alpha,
                             hipStream_t s) {
   if (rows == 0) return hipSuccess;
-  if (f <= 0 || kind < 0 || kind > 1) return hipErrorInvalidValue;
+  if (f <= 0 || kind < 0 || kind > 2) return hipErrorInvalidValue;
   hipLaunchKernelGGL(gated_act_kernel, dim3(rows), dim3(NT), 0, s, out, gu, f32, f, kind, limit, alpha);
   return hipGetLastError();
 }
@@ -415,6 +571,37 @@ hipError_t launch_topk_sigmoid(float* w, int* ids, const float* z, int T, int E,
   if (T == 0) return hipSuccess;
   if (E < 1 || E > ROUTE_E_MAX || K < 1 || K > E) return hipErrorInvalidValue;
   hipLaunchKernelGGL(topk_sigmoid_kernel, dim3((T + NT - 1) / NT), dim3(NT), 0, s, w, ids, z, T, E, K);
+  return hipGetLastError();
+}
+
+hipError_t launch_route_softmax_topk(float* w, int* ids, float* gate, const void* x, int64_t xstride, bool x_f32,
+                                     const void* wr, bool wr_f32, const float* corr, int T, int H, int E, int K,
+                                     hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  if (E < 1 || E > ROUTE_E_MAX || K < 1 || K > E) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(route_softmax_topk_kernel, dim3(T), dim3(NT), 0, s, w, ids, gate, x, xstride, x_f32, wr, wr_f32,
+                     corr, H, E, K);
+  return hipGetLastError();
+}
+
+hipError_t launch_topk_softmax_corrected(float* w, int* ids, float* gate, const float* z, int zstride,
+                                         const float* corr, int T, int E, int K, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  if (E < 1 || E > ROUTE_E_MAX || K < 1 || K > E || zstride < E + (gate ? 1 : 0)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(topk_softmax_corrected_kernel, dim3((T + SEL_NT - 1) / SEL_NT), dim3(SEL_NT),
+                     (size_t)SEL_NT * E * sizeof(float), s, w, ids, gate, z, zstride, corr, T, E, K);
+  return hipGetLastError();
+}
+
+hipError_t launch_combine_weighted(float* out, float* resid, void* act, const void* ys, bool f32, const int* pos,
+                                   const void* x, const float* wk, const int* ids, int E, const void* extra,
+                                   const float* gate, int T, int K, int H, const void* w, bool w_f32, bool unit_offset,
+                                   float eps, float mult, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  if (H <= 0 || H > 16384 || K < 1 || (out == nullptr && resid == nullptr) || (resid != nullptr && w == nullptr))
+    return hipErrorInvalidValue;
+  hipLaunchKernelGGL(combine_weighted_kernel, dim3(T), dim3(NT), (size_t)H * sizeof(float), s, out, resid, act, ys, f32,
+                     pos, x, wk, ids, E, extra, gate, K, H, w, w_f32, unit_offset, eps, mult);
   return hipGetLastError();
 }
 

@@ -90,6 +90,7 @@ struct QkvPrepArgs {
   const float* q_norm;    // [H * dim], [G * dim]: RMS norm over the whole projection, or nullptr
   const float* k_norm;
   bool head_norm;         // q_norm and k_norm are [dim], shared by all heads: RMS norm of every head by itself
+  bool norm_after_rot;    // with head_norm: the rotation comes first and the norm acts on the rotated heads
   float q_temp_coef;      // != 0: q, after its norm, times 1 + coef * ln(floor((p + 1) / q_temp_every) + 1) at position p
   int q_temp_every;
   int rot_dims;           // rotated dims per head (pairs i, i + rot_dims / 2), 0: none

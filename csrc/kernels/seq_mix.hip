@@ -626,6 +626,24 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
     }
   }
   const bool per_head = a.q_norm != nullptr && a.head_norm;
+  auto rotate = [&]() {
+    const int half = a.rot_dims / 2;
+    const float p = (float)a.positions[t];
+    for (int e = threadIdx.x; e < (H + G) * half; e += NT) {
+      const int hd = e / half, i = e % half;
+      float* base = hd < H ? qv + hd * d : kv + (hd - H) * d;
+      float sn, cs;
+      sincosf(p * a.inv_freq[i], &sn, &cs);
+      const float u = base[i], v = base[i + half];
+      base[i] = u * cs - v * sn;
+      base[i + half] = v * cs + u * sn;
+    }
+  };
+  const bool rot_first = per_head && a.norm_after_rot;
+  if (a.rot_dims > 0 && rot_first) {
+    __syncthreads();   // every thread's loads are in LDS
+    rotate();
+  }
   float qm = 1.0f;   // query temperature
   if (a.q_temp_coef != 0.f) {
     const int64_t p = a.positions[t];
@@ -668,19 +686,7 @@ __global__ void __launch_bounds__(NT) qkv_prep_kernel(QkvPrepArgs a) {
     for (int c = threadIdx.x; c < nq; c += NT) qv[c] *= qm;
     __syncthreads();
   }
-  if (a.rot_dims > 0) {
-    const int half = a.rot_dims / 2;
-    const float p = (float)a.positions[t];
-    for (int e = threadIdx.x; e < (H + G) * half; e += NT) {
-      const int hd = e / half, i = e % half;
-      float* base = hd < H ? qv + hd * d : kv + (hd - H) * d;
-      float sn, cs;
-      sincosf(p * a.inv_freq[i], &sn, &cs);
-      const float u = base[i], v = base[i + half];
-      base[i] = u * cs - v * sn;
-      base[i + half] = v * cs + u * sn;
-    }
-  }
+  if (a.rot_dims > 0 && !rot_first) rotate();
   if (a.v_unit) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int g = wave; g < G; g += NT / 64) {

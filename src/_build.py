@@ -95,8 +95,8 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False) -> 
     return out
 
 
-MIX_KERNELS = ["mix_ops", "latent_attn", "moe", "seq_mix", "sink_attn", "lin_mix"]
-MIX_BINDINGS = ["bindings_mix", "bindings_seq", "bindings_lin"]
+MIX_KERNELS = ["mix_ops", "latent_attn", "moe", "seq_mix", "sink_attn", "lin_mix", "rec_mix"]
+MIX_BINDINGS = ["bindings_mix", "bindings_seq", "bindings_lin", "bindings_rec"]
 # hipcc only: keeps -O3 from forming packed fp32 instructions out of ordinary float code
 NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

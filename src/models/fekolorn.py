@@ -59,6 +59,10 @@ class SinkAttnSpec:
     slope_exp: float = 0.0     # > 0: head h's score drops by 2^(-slope_exp (h + 1) / heads) per position of distance
     q_temp_coef: float = 0.0   # != 0: q times 1 + coef * ln(floor((p + 1) / q_temp_every) + 1) at position p
     q_temp_every: int = 1
+    rot_scaling: Optional[Tuple[float, float, float, float]] = None   # (factor, low, high, original): long
+    #                            wavelengths of the rotary frequencies stretched (src.ops.mix.rope_inv_freq)
+    norm_after_rot: bool = False   # with head_norm: the per-head norm follows the rotation instead of preceding it
+    norm_weights: bool = True      # False: the q / k norms have no weights (and the checkpoint no such tensors)
 
     @property
     def cache_width(self) -> int:
@@ -74,6 +78,8 @@ class SinkAttnSpec:
             c["mask"] = {"size": self.window}
         if self.rot_dims:
             c["rot"] = {"base": self.rot_base, "dims": self.rot_dims}
+            if self.rot_scaling is not None:
+                c["rot"]["scaling"] = dict(zip(("factor", "low", "high", "original"), self.rot_scaling))
         if self.bias_max:
             c["bias_max"] = self.bias_max
         if self.v_mix:
@@ -260,8 +266,14 @@ class SinkAttentionMixer:
         self.o = rnd(hidden, s.heads * s.vdim)
         f32 = torch.float32
         self.sink = rnd(s.heads, scale=0.5, dt=f32) if s.has_sink else None
-        self.q_norm = (1.0 + rnd(s.dim if s.head_norm else self.nq, scale=0.1, dt=f32)) if s.qk_norm else None
-        self.k_norm = (1.0 + rnd(s.dim if s.head_norm else self.nk, scale=0.1, dt=f32)) if s.qk_norm else None
+        if s.norm_after_rot and not s.head_norm:
+            raise ValueError("norm_after_rot is a form of head_norm")
+        nscale = 0.1 if s.norm_weights else 0.0   # weightless norms: ones that no checkpoint tensor replaces
+        self.q_norm = (1.0 + rnd(s.dim if s.head_norm else self.nq, scale=nscale, dt=f32)) if s.qk_norm else None
+        self.k_norm = (1.0 + rnd(s.dim if s.head_norm else self.nk, scale=nscale, dt=f32)) if s.qk_norm else None
+        if s.qk_norm and not s.norm_weights:
+            self.q_norm.fill_(1.0)
+            self.k_norm.fill_(1.0)
         # the distance penalty per head, rounded once from float64
         self.slopes = None
         if s.slope_exp:
@@ -273,7 +285,7 @@ class SinkAttentionMixer:
         self.rel_rows = max(2, min(32, 2 * (math.ceil(s.bias_max) - 1)))
         self.rel = rnd(self.rel_rows, s.heads, scale=0.5, dt=f32) if s.bias_max else None
         self.bias = None
-        self.inv_freq = mix.rope_inv_freq(s.rot_base, s.rot_dims, self.device) if s.rot_dims else None
+        self.inv_freq = mix.rope_inv_freq(s.rot_base, s.rot_dims, self.device, s.rot_scaling) if s.rot_dims else None
         self.finalize()
 
     def finalize(self) -> None:
@@ -298,9 +310,9 @@ class SinkAttentionMixer:
             return _put(self.o, t)
         if name == "sink" and self.sink is not None:
             return _put(self.sink, t)
-        if name == "q.norm" and self.q_norm is not None:
+        if name == "q.norm" and self.q_norm is not None and self.spec.norm_weights:
             return _put(self.q_norm, t)
-        if name == "k.norm" and self.k_norm is not None:
+        if name == "k.norm" and self.k_norm is not None and self.spec.norm_weights:
             return _put(self.k_norm, t)
         if name == "vmix" and self.vmix is not None:
             return _put(self.vmix, t)
@@ -316,7 +328,7 @@ class SinkAttentionMixer:
             out["v"] = self.qkv[self.nq + self.nk:]
         if self.sink is not None:
             out["sink"] = self.sink
-        if self.q_norm is not None:
+        if self.q_norm is not None and self.spec.norm_weights:
             out["q.norm"], out["k.norm"] = self.q_norm, self.k_norm
         if self.vmix is not None:
             out["vmix"] = self.vmix.reshape(())
@@ -339,7 +351,7 @@ class SinkAttentionMixer:
         qr = seq.qkv_prep(q, k, v, cache, s.heads, s.kv_heads, s.dim, s.vdim, positions, meta.slot_mapping, eps,
                           q_norm=self.q_norm, k_norm=self.k_norm, rot_dims=s.rot_dims, inv_freq=self.inv_freq,
                           v_unit=s.v_unit, v_lambda=lam, v_first=v_first, head_norm=s.head_norm,
-                          q_temp_coef=s.q_temp_coef, q_temp_every=s.q_temp_every)
+                          q_temp_coef=s.q_temp_coef, q_temp_every=s.q_temp_every, norm_after_rot=s.norm_after_rot)
         o = seq.sink_attn(qr, cache, meta.block_tables, meta.cu_q if meta.is_prefill else None, meta.ctx_lens,
                           positions, self.sink, self.bias, meta.max_q_len if meta.is_prefill else 1, s.heads,
                           s.kv_heads, s.dim, s.vdim, s.window, s.scale, softcap=s.softcap, slopes=self.slopes)

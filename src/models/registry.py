@@ -6,7 +6,9 @@ Model-class registry: which model class serves a checkpoint directory, decided b
 * ``"architecture": "Fekolorn"`` (layers listed in the config, per-sequence state) ->
   :class:`src.models.fekolorn.FekolornLM`;
 * ``"architecture": "Bapivik"`` (layers listed in the config, learned positions, depth-averaged layer results) ->
-  :class:`src.models.bapivik.BapivikLM`.
+  :class:`src.models.bapivik.BapivikLM`;
+* ``"architecture": "Kogerax"`` (layers listed in the config: matrix-memory LSTM, scalar-decay state space, attention
+  beside a selective scan; unnormed sublayer inputs, normed outputs) -> :class:`src.models.kogerax.KogeraxLM`.
 
 A new family registers a (matcher, arch reader, model class) triple with :func:`register_family`.
 """
@@ -101,8 +103,21 @@ def _bapivik_arch(path: str, **kw):
     return bapivik_arch_from_dir(path, **kw)
 
 
+def _kogerax_cls():
+    from src.models.kogerax import KogeraxLM
+
+    return KogeraxLM
+
+
+def _kogerax_arch(path: str, **kw):
+    from src.models.kogerax import kogerax_arch_from_dir
+
+    return kogerax_arch_from_dir(path, **kw)
+
+
 register_family("datatar", lambda c: c.get("architecture") == "Datatar", _datatar_arch, _datatar_cls)
 register_family("fekolorn", lambda c: c.get("architecture") == "Fekolorn", _fekolorn_arch, _fekolorn_cls)
 register_family("bapivik", lambda c: c.get("architecture") == "Bapivik", _bapivik_arch, _bapivik_cls)
+register_family("kogerax", lambda c: c.get("architecture") == "Kogerax", _kogerax_arch, _kogerax_cls)
 register_family("llama", lambda c: "architecture" not in c and c.get("model_type", "llama") in
                 ("llama", "mistral", "mixtral"), _llama_arch, _llama_cls)

@@ -15,6 +15,7 @@ semantics in :mod:`src.ops.reference`, which lets the engine's control flow run 
 
 from __future__ import annotations
 
+import math
 from typing import Optional, Tuple
 
 import torch
@@ -68,24 +69,25 @@ def rms_norm_ext(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, unit_of
 
 
 def post_norm_residual(resid: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float, unit_offset: bool = True,
-                       act: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """resid (fp32 [rows, n], in place) += rmsnorm(y) * g — the norm sits on the sublayer's output, the residual
-    sum is fp32. ``act`` (bf16, same shape): also receives the new residual, the next projection's input."""
+                       act: Optional[torch.Tensor] = None, mult: float = 1.0) -> torch.Tensor:
+    """resid (fp32 [rows, n], in place) += mult * rmsnorm(y) * g — the norm sits on the sublayer's output, the
+    residual sum is fp32. ``act`` (bf16, same shape): also receives the new residual, the next projection's input."""
     if not resid.is_cuda:
-        resid.add_(ref.rms_norm_ext(y, w, eps, unit_offset, torch.float32))
+        resid.add_(ref.rms_norm_ext(y, w, eps, unit_offset, torch.float32), alpha=mult)
         if act is not None:
             act.copy_(resid)
         return resid
-    _kern().post_norm_residual(resid, act, y, w, unit_offset, eps)
+    _kern().post_norm_residual(resid, act, y, w, unit_offset, eps, float(mult))
     return resid
 
 
-ACT_SILU, ACT_CLAMPED = 0, 1
+ACT_SILU, ACT_CLAMPED, ACT_GELU_TANH = 0, 1, 2
 
 
 def gated_act(gu: torch.Tensor, kind: int = ACT_SILU, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
     """[rows, 2f] = [gate | up] -> [rows, f]. ACT_SILU: silu(g) * u. ACT_CLAMPED: g' = min(g, limit),
-    u' = clamp(u, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1)."""
+    u' = clamp(u, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1). ACT_GELU_TANH: gelu(g) * u with the tanh
+    form 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3)))."""
     if not gu.is_cuda:
         return ref.gated_act(gu, kind, limit, alpha)
     gu = gu.contiguous()
@@ -202,10 +204,105 @@ def moe_input_scaled(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w: to
     return finish(ys, pos)
 
 
-def rope_inv_freq(base: float, dims: int, device) -> torch.Tensor:
-    """fp32 [dims / 2]: base^(-2 i / dims), rounded once from float64."""
+def route_softmax_topk(x: torch.Tensor, router: torch.Tensor, k: int, n_route: int,
+                       correction: Optional[torch.Tensor] = None, gate_row: bool = False):
+    """Softmax-scored routing over ``n_route`` choices (fp32 logits x . router[e], e < n_route): the k largest
+    scores + correction (lowest index on ties) are chosen; their weights are the scores WITHOUT the correction,
+    divided by their sum (+ 1e-20). With ``gate_row`` the router has one more row whose logit goes through a sigmoid
+    (a per-token gate that rides in the same product). Returns (w [T, k] fp32, ids [T, k] int32, gate [T] fp32 or
+    None)."""
+    t = x.shape[0]
+    rows = n_route + (1 if gate_row else 0)
+    if not x.is_cuda:
+        z = x.float() @ router[:rows].float().t()
+        w, ids = ref.softmax_topk_corrected(z[:, :n_route], k, correction)
+        return w, ids, (torch.sigmoid(z[:, n_route]).contiguous() if gate_row else None)
+    w = torch.empty(t, k, dtype=torch.float32, device=x.device)
+    ids = torch.empty(t, k, dtype=torch.int32, device=x.device)
+    gate = torch.empty(t, dtype=torch.float32, device=x.device) if gate_row else None
+    if t > ROUTE_FUSED_MAX_T:
+        # prompt-sized steps: the logits as one true-fp32 library GEMM, then the selection kernel
+        _kern().topk_softmax_corrected(w, ids, gate, F.linear(x.float(), router[:rows].float()), n_route, correction)
+    else:
+        _kern().route_softmax_topk(w, ids, gate, x, router.contiguous(), n_route, correction)
+    return w, ids, gate
+
+
+def moe_output_weighted(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w: torch.Tensor, ids: torch.Tensor,
+                        kind: int, limit: float, alpha: float, n_route: int = 0,
+                        extra: Optional[torch.Tensor] = None, extra_gate: Optional[torch.Tensor] = None,
+                        post_norm=None) -> Optional[torch.Tensor]:
+    """out[t] (fp32) = sum_j w[t, j] * expert_{ids[t, j]}(x[t]) (+ extra_gate[t] * extra[t]); expert(z) =
+    W2 act(W1 z, W3 z) with w13 [E, 2f, H] = [W1; W3], w2 [E, H, f] and ``act`` one of :func:`gated_act`'s kinds. An
+    id in [E, n_route) names an identity expert, whose output is x[t] itself. The routing weight multiplies the expert's OUTPUT
+    (in fp32, in the launch that sums). ``post_norm`` = (resid fp32 [T, H], norm weight, eps, unit_offset, act or
+    None, mult): instead of returning the sum, add mult * its RMS-normalised form into ``resid`` (and refresh ``act``)
+    in the same launch; returns None."""
+    if not x.is_cuda:
+        out = ref.moe_output_weighted(x, w13, w2, w, ids, kind, limit, alpha, extra, extra_gate)
+        if post_norm is None:
+            return out
+        resid, nw, eps, unit, act, mult = post_norm
+        post_norm_residual(resid, out, nw, eps, unit, act=act, mult=mult)
+        return None
+    kern = _kern()
+    t, h = x.shape
+    k = ids.shape[1]
+    n = t * k
+    e = w13.shape[0]
+    x = x.contiguous()
+    w = w.contiguous()
+
+    def finish(ys, pos):
+        if post_norm is not None:
+            resid, nw, eps, unit, act, mult = post_norm
+            kern.combine_weighted(None, resid, act, ys, pos, x, w, ids, e, extra, extra_gate, nw, unit, eps, float(mult))
+            return None
+        out = torch.empty(t, h, dtype=torch.float32, device=x.device)
+        kern.combine_weighted(out, None, None, ys, pos, x, w, ids, e, extra, extra_gate, None, False, 0.0, 1.0)
+        return out
+
+    if e == 0:
+        return finish(torch.empty(0, h, dtype=x.dtype, device=x.device), None)
+    if n <= MOE_BMM_MAX_ROWS or torch.cuda.is_current_stream_capturing():
+        # decode-sized steps: the routed experts' weights gathered per row for two batched products (no host read,
+        # hipGraph-capturable); an identity entry runs expert E - 1 and its product is ignored by the sum
+        sel = ids.reshape(-1).long().clamp_(max=e - 1)
+        xr = x.unsqueeze(1).expand(t, k, h).reshape(n, h, 1)
+        g = torch.bmm(w13.index_select(0, sel), xr).squeeze(2)
+        ys = torch.bmm(w2.index_select(0, sel), gated_act(g, kind, limit, alpha).unsqueeze(2)).squeeze(2).contiguous()
+        return finish(ys, None)
+    # prompt-sized steps: rows sorted by expert (identity entries sort last and run nothing), one library GEMM pair
+    # per real expert over its rows
+    buckets = max(e, int(n_route))
+    offsets = torch.empty(buckets + 1, dtype=torch.int32, device=x.device)
+    sorted_idx = torch.empty(n, dtype=torch.int32, device=x.device)
+    pos = torch.empty(n, dtype=torch.int32, device=x.device)
+    kern.moe_align(offsets, sorted_idx, pos, ids.reshape(-1).contiguous(), buckets)
+    xs = torch.empty(n, h, dtype=x.dtype, device=x.device)
+    kern.gather_scaled(xs, x, sorted_idx, None, k)
+    ys = torch.empty(n, h, dtype=x.dtype, device=x.device)
+    off = offsets.tolist()  # one host read per layer: the per-expert groups become library GEMMs
+    for ei in range(e):
+        a0, a1 = off[ei], off[ei + 1]
+        if a1 > a0:
+            F.linear(gated_act(F.linear(xs[a0:a1], w13[ei]), kind, limit, alpha), w2[ei], out=ys[a0:a1])
+    return finish(ys, pos)
+
+
+def rope_inv_freq(base: float, dims: int, device, scaling: Optional[Tuple[float, float, float, float]] = None) -> torch.Tensor:
+    """fp32 [dims / 2]: base^(-2 i / dims), rounded once from float64. ``scaling`` = (factor, low, high, original)
+    stretches long wavelengths: with l = 2 pi / f, f stays where l < original / high, becomes f / factor where
+    l > original / low, and in between (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
     i = torch.arange(dims // 2, dtype=torch.float64)
-    return (float(base) ** (-2.0 * i / dims)).float().to(device)
+    f = float(base) ** (-2.0 * i / dims)
+    if scaling is not None:
+        factor, low, high, orig = (float(v) for v in scaling)
+        wl = 2.0 * math.pi / f
+        s = (orig / wl - low) / (high - low) if high != low else torch.ones_like(f)
+        mid = (1.0 - s) * f / factor + s * f
+        f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, mid))
+    return f.float().to(device)
 
 
 def latent_kv_write(cache: torch.Tensor, kv: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,

@@ -185,6 +185,9 @@ def gated_act(gu: torch.Tensor, kind: int, limit: float, alpha: float) -> torch.
     g, u = gu[..., :f].float(), gu[..., f:].float()
     if kind == 0:
         return (g * torch.sigmoid(g) * u).to(gu.dtype)
+    if kind == 2:
+        gg = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
+        return (gg * u).to(gu.dtype)
     g = torch.clamp(g, max=limit)
     u = torch.clamp(u, -limit, limit)
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
@@ -205,6 +208,34 @@ def moe_input_scaled(x, w13, w2, w, ids, extra=None) -> torch.Tensor:
             xs = (w[rows, j, None] * x[rows].float()).to(x.dtype)
             a = gated_act(torch.nn.functional.linear(xs, w13[e]), 0, 0.0, 1.0)
             out[rows] += torch.nn.functional.linear(a, w2[e]).float()
+    return out
+
+
+def softmax_topk_corrected(z: torch.Tensor, k: int, correction: Optional[torch.Tensor]):
+    """z [T, E] fp32 logits: the k largest softmax(z) + correction (lowest index on ties); weights = the chosen
+    scores without the correction, over their sum + 1e-20."""
+    s = torch.softmax(z.float(), -1)
+    c = s if correction is None else s + correction.float()
+    ids = torch.sort(c, dim=-1, descending=True, stable=True).indices[:, :k]
+    w = torch.gather(s, 1, ids)
+    return (w / (w.sum(-1, keepdim=True) + 1e-20)).contiguous(), ids.to(torch.int32).contiguous()
+
+
+def moe_output_weighted(x, w13, w2, w, ids, kind, limit, alpha, extra=None, extra_gate=None) -> torch.Tensor:
+    t, h = x.shape
+    e_real = w13.shape[0]
+    out = torch.zeros(t, h, dtype=torch.float32)
+    for j in range(ids.shape[1]):
+        for e in ids[:, j].unique().tolist():
+            rows = (ids[:, j] == e).nonzero().flatten()
+            if e >= e_real:
+                y = x[rows].float()
+            else:
+                a = gated_act(torch.nn.functional.linear(x[rows], w13[e]), kind, limit, alpha)
+                y = torch.nn.functional.linear(a, w2[e]).float()
+            out[rows] += w[rows, j, None] * y
+    if extra is not None:
+        out += extra.float() if extra_gate is None else extra_gate[:, None] * extra.float()
     return out
 
 

@@ -256,12 +256,13 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], cache:
              q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None, rot_dims: int = 0,
              inv_freq: Optional[torch.Tensor] = None, v_unit: bool = False, v_lambda: Optional[torch.Tensor] = None,
              v_first: Optional[torch.Tensor] = None, head_norm: bool = False, q_temp_coef: float = 0.0,
-             q_temp_every: int = 1) -> torch.Tensor:
+             q_temp_every: int = 1, norm_after_rot: bool = False) -> torch.Tensor:
     """The step between the q/k/v projection and the attention, one launch: optional RMS norm of q and of k (plain
     weights) over the whole projection or, with ``head_norm``, of every head by itself with weights [dim] shared by
     the heads; optional query temperature, q times 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1) after its
     norm; optional rotate-half rotary on the first ``rot_dims`` dims of every head (pair i, i + rot_dims / 2, angle
-    position * inv_freq[i]); values either divided by their per-head root mean square or blended as
+    position * inv_freq[i]) — with ``norm_after_rot`` (and ``head_norm``) the rotation comes first and the per-head
+    norm acts on the rotated heads; values either divided by their per-head root mean square or blended as
     (1 - l) v + l v_first; ``v`` None: the values are the keys as projected, before norm and rotation. Writes the
     token's keys and values into the cache at slots[t] (< 0: skipped; a block's interior is head-major,
     [G][block_size][k | v]) and returns q [T, H * dim]."""
@@ -269,13 +270,27 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], cache:
     if q.is_cuda:
         q_out = torch.empty(T, heads * dim, dtype=q.dtype, device=q.device)
         _kern().qkv_prep(q_out, cache, q, k, v, heads, kv_heads, dim, vdim, q_norm, k_norm, rot_dims, inv_freq, v_unit,
-                         v_lambda, v_first, eps, positions, slots, head_norm, float(q_temp_coef), int(q_temp_every))
+                         v_lambda, v_first, eps, positions, slots, head_norm, float(q_temp_coef), int(q_temp_every),
+                         bool(norm_after_rot))
         return q_out
     if v is None:
         v = k
     qf, kf, vf = q.float(), k.float(), v.float()
     if v_lambda is not None:
         vf = (1.0 - v_lambda) * vf + v_lambda * v_first.float()
+
+    def rot(x, n):
+        half = rot_dims // 2
+        ang = positions.float()[:, None] * inv_freq[None, :]
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        x = x.view(T, n, dim).clone()
+        u, w = x[..., :half].clone(), x[..., half:rot_dims].clone()
+        x[..., :half] = u * c - w * s
+        x[..., half:rot_dims] = w * c + u * s
+        return x.reshape(T, n * dim)
+
+    if rot_dims and norm_after_rot:
+        qf, kf = rot(qf, heads), rot(kf, kv_heads)
     if q_norm is not None and head_norm:
         qh, kh = qf.view(T, heads, dim), kf.view(T, kv_heads, dim)
         qf = (qh / torch.sqrt((qh * qh).mean(-1, keepdim=True) + eps) * q_norm).reshape(T, heads * dim)
@@ -286,18 +301,7 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], cache:
     if q_temp_coef:
         steps = torch.div(positions + 1, q_temp_every, rounding_mode="floor").float()
         qf = qf * (1.0 + q_temp_coef * torch.log(steps + 1.0))[:, None]
-    if rot_dims:
-        half = rot_dims // 2
-        ang = positions.float()[:, None] * inv_freq[None, :]
-        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
-
-        def rot(x, n):
-            x = x.view(T, n, dim).clone()
-            u, w = x[..., :half].clone(), x[..., half:rot_dims].clone()
-            x[..., :half] = u * c - w * s
-            x[..., half:rot_dims] = w * c + u * s
-            return x.reshape(T, n * dim)
-
+    if rot_dims and not norm_after_rot:
         qf, kf = rot(qf, heads), rot(kf, kv_heads)
     if v_unit:
         vh = vf.view(T, kv_heads, vdim)

@@ -60,7 +60,7 @@ def main(argv=None) -> int:
     from src.models.registry import family_of
 
     family = family_of(a.model)
-    generic = family in ("datatar", "fekolorn", "bapivik")   # families on the dtype-generic kernels (src/_Cmix) alone
+    generic = family in ("datatar", "fekolorn", "bapivik", "kogerax")   # families on the dtype-generic kernels (src/_Cmix) alone
     if not generic and a.dtype == "float32":
         print(f"the {family} kernels are bfloat16 only", file=sys.stderr)
         return 3
