@@ -356,3 +356,73 @@ def make_weights(config: Dict[str, Any], seed: int = 0, dtype=torch.float32) -> 
             t = torch.randn(shape, generator=g) * (1.5 / math.sqrt(shape[-1]))
         out[name] = t.to(torch.bfloat16).to(dtype)
     return out
+
+
+def routing_margins(config: Dict[str, Any], weights: Dict[str, torch.Tensor], tokens: List[int]) -> torch.Tensor:
+    """Per position: the smallest gap, over all mixture layers, between the last chosen and the first rejected choice
+    score. A position whose gap is below the compared precision may legitimately route differently."""
+    W = {k: v.to(F64) for k, v in weights.items()}
+    eps = float(config["norm"]["eps"])
+    mult = float(config.get("residual_mult", 1.0))
+
+    def sub(prefix):
+        return {k[len(prefix):]: v for k, v in W.items() if k.startswith(prefix)}
+
+    x = W["embed"][torch.tensor(tokens)] * float((config.get("embedding") or {}).get("scale", 1.0))
+    gaps = torch.full((len(tokens),), math.inf, dtype=F64)
+    for i, lc in enumerate(config["layers"]):
+        p = f"l{i}."
+        x = x + mult * rms(MIXERS[lc["type"]](x, sub(p + "mix."), lc["mixer"], eps), eps) * (1.0 + W[p + "norm1"])
+        f = lc.get("mlp")
+        if f is None:
+            continue
+        if f["kind"] == "moe":
+            w = sub(p + "mlp.")
+            s = torch.softmax(x @ w["router"].T, -1)
+            c = torch.sort(s + w["correction"], -1, descending=True).values
+            k = int(f["router"]["top"])
+            if k < c.shape[1]:
+                gaps = torch.minimum(gaps, c[:, k - 1] - c[:, k])
+        x = x + mult * rms(feed_forward(x, sub(p + "mlp."), f), eps) * (1.0 + W[p + "norm2"])
+    return gaps
+
+
+# layer entries of a configuration
+def dense(ff: int = 40) -> Dict[str, Any]:
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts: int = 4, identity: int = 2, top: int = 3, ff: int = 24, limit: float = 1.5, shared_ff: int = 16,
+        shared_limit: float = 2.5) -> Dict[str, Any]:
+    f: Dict[str, Any] = {"kind": "moe", "expert": {"ff": ff, "limit": limit},
+                         "router": {"experts": experts, "identity": identity, "top": top}}
+    if shared_ff:
+        f["shared"] = {"ff": shared_ff, "limit": shared_limit}
+    return f
+
+
+def mlstm_layer(heads=2, dim=8, vdim=12, gate_cap=10.0, mlp=None) -> Dict[str, Any]:
+    return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "gate_cap": gate_cap}, "mlp": mlp}
+
+
+def mamba2_layer(heads=4, vdim=6, state=8, groups=2, conv=4, norm_groups=2, mlp=None) -> Dict[str, Any]:
+    return {"type": "mamba2", "mixer": {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv,
+                                        "norm_groups": norm_groups}, "mlp": mlp}
+
+
+def parallel_layer(heads=4, kv_heads=2, dim=16, vdim=8, window=9, rot_dims=8, rot_base=100.0, scaling=(8.0, 1.0, 4.0, 40),
+                   scale=0.4, inner=24, state=6, dt_rank=3, conv=3, mlp=None) -> Dict[str, Any]:
+    left: Dict[str, Any] = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if window:
+        left["mask"] = {"size": window}
+    if rot_dims:
+        left["rot"] = {"base": rot_base, "dims": rot_dims}
+        if scaling:
+            left["rot"]["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
+    right = {"inner": inner, "state": state, "dt_rank": dt_rank, "conv": conv}
+    return {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp}
+
+
+def make_config(layers, vocab=67, width=32, eps=1e-5, embed_scale=3.0, residual_mult=0.4) -> Dict[str, Any]:
+    return {"architecture": "Kogerax", "embedding": {"scale": embed_scale}, "layers": layers, "norm": {"eps": eps},
+            "residual_mult": residual_mult, "vocab": vocab, "width": width}
