@@ -268,7 +268,10 @@ def _mixer_case(device, kind, spec_cfg, dt=torch.float32, W=24, seed=0):
     for s in range(2):
         assert got[s].shape[0] == at[s]
         ref = want[s][: at[s]]
-        assert float((got[s] - ref).abs().max()) < tol * float(ref.abs().max()), (kind, s)
+        if dt == torch.float32:
+            assert float((got[s] - ref).abs().max()) < tol * float(ref.abs().max()), (kind, s)
+        else:   # bf16: a norm over a narrow part of the row magnifies single rounding errors; the whole is held
+            assert float((got[s] - ref).pow(2).mean().sqrt()) < tol * float(ref.pow(2).mean().sqrt()), (kind, s)
     for t in state.values():
         if t.numel() == 0:       # a one-tap convolution keeps no tail
             continue
@@ -393,7 +396,7 @@ def test_attention_window_edges_and_far_keys(device, where, rows):
         if where == "outside":
             assert moved < 1e-9
         else:
-            assert moved > 100 * tol * float(want.abs().max())
+            assert moved > 0.5 * float(want.abs().max())   # the key carries the last row's output
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -624,11 +627,13 @@ def test_greedy_generation_through_the_engine(tmp_path, device):
     n_new = 6
 
     def is_greedy(prompt, out):
-        """Every generated token is the oracle's argmax given the tokens before it (or within a rounding error)."""
+        """Every generated token is the oracle's argmax given the tokens before it, or ties with it at the sampler's
+        precision (the GPU sampling kernel reads the logits as bf16)."""
         seq_ = list(prompt)
         for tok in out:
             lg = orc.forward(config, weights, seq_)[-1]
-            if float(lg[tok]) < float(lg.max()) - 1e-3 * float(lg.std()):
+            slack = 1e-3 * float(lg.std()) if device == "cpu" else 2.0 ** -7 * float(lg.abs().max())
+            if float(lg[tok]) < float(lg.max()) - slack:
                 return False
             seq_.append(tok)
         return len(out) == n_new
