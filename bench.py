@@ -135,6 +135,10 @@ def parse(argv=None):
                    help="instead of the serving benchmark: the Bapivik design beside Llama at equal "
                         "sizes, prefill / decode throughput and its kernels alone (bench/bapivik_compare.py)")
     p.add_argument("--bapivik-args", default="", help="arguments passed on to bench/bapivik_compare.py")
+    p.add_argument("--kogerax-compare", action="store_true",
+                   help="instead of the default workload: Kogerax beside Fekolorn (recurrent state next to attention) at "
+                        "equal sizes, prefill / decode throughput and its kernels alone (bench/kogerax_compare.py)")
+    p.add_argument("--kogerax-args", default="", help="arguments passed on to bench/kogerax_compare.py")
     return p.parse_args(argv)
 
 
@@ -492,6 +496,15 @@ def main(argv=None) -> int:
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
         return mod.main(shlex.split(args.bapivik_args))
+    if args.kogerax_compare:  # likewise a separate measurement
+        import importlib.util
+        import shlex
+
+        spec = importlib.util.spec_from_file_location("kogerax_compare",
+                                                      os.path.join(ROOT, "bench", "kogerax_compare.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        return mod.main(shlex.split(args.kogerax_args))
     if needs_launcher(args):
         return self_launch(args, argv)
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -205,7 +205,15 @@ constexpr int SCH = 256; // threads per workgroup of the scan
 // in registers for the whole step; a token costs a lane NP exponentials and 3 NP multiply-adds, plus a reduction
 // over the LPC lanes. B_t and C_t come from LDS as float4 broadcasts; x, step size and z of TB tokens are staged
 // per trip.
-template <int NP, int LPC>
+// exp(d * A): fp32 steps use expf; bf16 steps fold log2(e) into A once and use the hardware's 2^x (v_exp_f32)
+template <bool FAST> __device__ __forceinline__ float decay_of(float d, float a) {
+  if constexpr (FAST)
+    return __builtin_amdgcn_exp2f(d * a);
+  else
+    return expf(d * a);
+}
+
+template <int NP, int LPC, bool FAST>
 __global__ void __launch_bounds__(SCH) selective_scan_kernel(SelectiveScanArgs a, RaggedRows r) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   constexpr int NPAD = NP * LPC, CH = SCH / LPC;
@@ -231,7 +239,7 @@ __global__ void __launch_bounds__(SCH) selective_scan_kernel(SelectiveScanArgs a
     const int n = part * NP + i;
     const bool ok = live && n < N;
     S[i] = (ok && !fresh) ? st[n] : 0.f;
-    A[i] = ok ? a.A[(int64_t)c * N + n] : 0.f;
+    A[i] = ok ? a.A[(int64_t)c * N + n] * (FAST ? 1.4426950408889634f : 1.0f) : 0.f;
   }
   const float Dc = live ? a.D[c] : 0.f;
   for (int t0 = 0; t0 < L; t0 += TB) {
@@ -261,10 +269,10 @@ __global__ void __launch_bounds__(SCH) selective_scan_kernel(SelectiveScanArgs a
 #pragma unroll
       for (int i = 0; i < NP / 4; ++i) {
         const float4 b4 = Bt[i], c4 = Ct[i];
-        S[4 * i] = expf(d * A[4 * i]) * S[4 * i] + dx * b4.x;
-        S[4 * i + 1] = expf(d * A[4 * i + 1]) * S[4 * i + 1] + dx * b4.y;
-        S[4 * i + 2] = expf(d * A[4 * i + 2]) * S[4 * i + 2] + dx * b4.z;
-        S[4 * i + 3] = expf(d * A[4 * i + 3]) * S[4 * i + 3] + dx * b4.w;
+        S[4 * i] = decay_of<FAST>(d, A[4 * i]) * S[4 * i] + dx * b4.x;
+        S[4 * i + 1] = decay_of<FAST>(d, A[4 * i + 1]) * S[4 * i + 1] + dx * b4.y;
+        S[4 * i + 2] = decay_of<FAST>(d, A[4 * i + 2]) * S[4 * i + 2] + dx * b4.z;
+        S[4 * i + 3] = decay_of<FAST>(d, A[4 * i + 3]) * S[4 * i + 3] + dx * b4.w;
         y0 += S[4 * i] * c4.x + S[4 * i + 2] * c4.z;
         y1 += S[4 * i + 1] * c4.y + S[4 * i + 3] * c4.w;
       }
@@ -289,7 +297,11 @@ __global__ void __launch_bounds__(SCH) selective_scan_kernel(SelectiveScanArgs a
 template <int NP, int LPC> hipError_t launch_scan_one(const SelectiveScanArgs& a, RaggedRows r, hipStream_t s) {
   constexpr int CH = SCH / LPC;
   const size_t smem = (size_t)TB * (2 * NP * LPC + 3 * CH) * sizeof(float);
-  hipLaunchKernelGGL((selective_scan_kernel<NP, LPC>), dim3((a.I + CH - 1) / CH, r.num_seqs), dim3(SCH), smem, s, a, r);
+  const dim3 grid((a.I + CH - 1) / CH, r.num_seqs);
+  if (a.f32)
+    hipLaunchKernelGGL((selective_scan_kernel<NP, LPC, false>), grid, dim3(SCH), smem, s, a, r);
+  else
+    hipLaunchKernelGGL((selective_scan_kernel<NP, LPC, true>), grid, dim3(SCH), smem, s, a, r);
   return hipGetLastError();
 }
 
@@ -339,24 +351,26 @@ __global__ void __launch_bounds__(64) exp_gate_scan_kernel(float* abe, const voi
 }
 
 // ---------------------------------------------------------------------------------------- matrix recurrence
-// One workgroup per (head, sequence, block of VC columns); blockIdx.z == the number of column blocks handles the
-// normaliser vector as one more column whose value is 1. The state lives in registers for the whole step: column j
-// is split over the 4 lanes of a quad, lane `part` holding rows [part * DP, (part + 1) * DP). A token costs each lane
-// 2 * DP multiply-adds and one quad reduction; q (scaled) and b * k come from LDS as float4 broadcasts.
+// One workgroup per (head, sequence, block of VC columns). The state lives in registers for the whole step: column j
+// is split over the 4 lanes of a quad, lane `part` holding rows [part * DP, (part + 1) * DP). With a normaliser, column
+// block 0 carries it as one more column (the quad after the last value column) whose value is 1. A token costs each
+// lane 2 * DP multiply-adds and one quad reduction; q (scaled) and k come from LDS as float4 broadcasts, b scales the
+// value.
 template <int DP>
-__global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs a, RaggedRows r, int VC, int nvc) {
+__global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs a, RaggedRows r, int VC) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   constexpr int DPAD = 4 * DP;
   const int d = a.dim, dv = a.vdim, H = a.heads;
   float* qs = sm;                  // [TB][DPAD], zero beyond dim
-  float* ks = qs + TB * DPAD;      // [TB][DPAD], already times b
+  float* ks = qs + TB * DPAD;      // [TB][DPAD]
   float* vs = ks + TB * DPAD;      // [TB][VC]
-  float* as = vs + TB * VC;        // [TB]
+  float* as = vs + TB * VC;        // [TB][2]: a, b
   const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x, nthr = blockDim.x;
-  const bool is_n = (int)blockIdx.z == nvc;
-  const int v0 = is_n ? 0 : blockIdx.z * VC;
-  const int ncol = is_n ? 1 : min(VC, dv - v0);
+  const int v0 = blockIdx.z * VC;
+  const int ncol = min(VC, dv - v0);
   const int j = tid >> 2, part = tid & 3;
+  const bool is_n = a.n_state != nullptr && blockIdx.z == 0 && j == ncol;   // this quad holds the normaliser
+  const bool used = j < ncol || is_n;
   const int g = h / (H / a.groups);
   const int q0 = r.cu_q ? r.cu_q[s] : s;
   const int L = r.cu_q ? r.cu_q[s + 1] - q0 : 1;
@@ -371,32 +385,29 @@ __global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs
 #pragma unroll
   for (int i = 0; i < DP; ++i) {
     const int row = part * DP + i;
-    S[i] = (!fresh && row < d && j < ncol) ? st[(int64_t)row * rs] : 0.f;
+    S[i] = (!fresh && row < d && used) ? st[(int64_t)row * rs] : 0.f;
   }
   for (int t0 = 0; t0 < L; t0 += TB) {
     const int nb = min(TB, L - t0);
     __syncthreads();
     for (int e = tid; e < nb * DPAD; e += nthr) {
       const int tt = e / DPAD, c = e % DPAD;
-      const int64_t row = q0 + t0 + tt;
-      const int64_t base = row * a.xstride + g * d + c;
-      const float b = a.ab[(row * H + h) * a.abw + 1];
+      const int64_t base = (int64_t)(q0 + t0 + tt) * a.xstride + g * d + c;
       qs[e] = c < d ? ldv(a.x, base + a.qoff, f32) * a.qscale : 0.f;
-      ks[e] = c < d ? ldv(a.x, base + a.koff, f32) * b : 0.f;
+      ks[e] = c < d ? ldv(a.x, base + a.koff, f32) : 0.f;
     }
-    if (!is_n) {
-      for (int e = tid; e < nb * VC; e += nthr) {
-        const int tt = e / VC, c = e % VC;
-        vs[e] = c < ncol ? ldv(a.x, (int64_t)(q0 + t0 + tt) * a.xstride + a.voff + h * dv + v0 + c, f32) : 0.f;
-      }
+    for (int e = tid; e < nb * VC; e += nthr) {
+      const int tt = e / VC, c = e % VC;
+      vs[e] = c < ncol ? ldv(a.x, (int64_t)(q0 + t0 + tt) * a.xstride + a.voff + h * dv + v0 + c, f32) : 0.f;
     }
-    for (int e = tid; e < nb; e += nthr) as[e] = a.ab[((int64_t)(q0 + t0 + e) * H + h) * a.abw];
+    for (int e = tid; e < 2 * nb; e += nthr) as[e] = a.ab[((int64_t)(q0 + t0 + (e >> 1)) * H + h) * a.abw + (e & 1)];
     __syncthreads();
     for (int tt = 0; tt < nb; ++tt) {
       const float4* kt = reinterpret_cast<const float4*>(ks + tt * DPAD + part * DP);
       const float4* qt = reinterpret_cast<const float4*>(qs + tt * DPAD + part * DP);
-      const float vj = is_n ? 1.0f : (j < ncol ? vs[tt * VC + j] : 0.f);
-      const float dec = as[tt];
+      const float2 ab = *reinterpret_cast<const float2*>(as + 2 * tt);
+      const float vj = (is_n ? 1.0f : (j < ncol ? vs[tt * VC + j] : 0.f)) * ab.y;
+      const float dec = ab.x;
       float o0 = 0.f, o1 = 0.f;
 #pragma unroll
       for (int i = 0; i < DP / 4; ++i) {
@@ -411,7 +422,7 @@ __global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs
       float o = o0 + o1;
       o += __shfl_xor(o, 1, 64);
       o += __shfl_xor(o, 2, 64);
-      if (part == 0 && j < ncol) {
+      if (part == 0 && used) {
         const int64_t row = q0 + t0 + tt;
         if (is_n)
           a.nq[row * H + h] = o;
@@ -420,7 +431,7 @@ __global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs
       }
     }
   }
-  if (j < ncol) {
+  if (used) {
 #pragma unroll
     for (int i = 0; i < DP; ++i) {
       const int row = part * DP + i;
@@ -432,68 +443,177 @@ __global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs
 template <int DP> hipError_t launch_gla_dp(const GatedLinearArgs& a, RaggedRows r, hipStream_t s) {
   const int VC = a.vdim < 128 ? a.vdim : 128;
   const int nvc = (a.vdim + VC - 1) / VC;
-  const int threads = (4 * VC + 63) / 64 * 64;
-  const size_t smem = (size_t)(2 * TB * 4 * DP + TB * VC + TB) * sizeof(float);
-  hipLaunchKernelGGL(gated_linear_attn_kernel<DP>, dim3(a.heads, r.num_seqs, nvc + (a.n_state ? 1 : 0)), dim3(threads),
-                     smem, s, a, r, VC, nvc);
+  const int threads = (4 * (VC + (a.n_state ? 1 : 0)) + 63) / 64 * 64;
+  const size_t smem = (size_t)(2 * TB * 4 * DP + TB * VC + 2 * TB) * sizeof(float);
+  hipLaunchKernelGGL(gated_linear_attn_kernel<DP>, dim3(a.heads, r.num_seqs, nvc), dim3(threads), smem, s, a, r, VC);
   return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------------ epilogues
-// One workgroup per token, a wave per head at a time.
+// 4 consecutive activations (element index a multiple of 4, 8- / 16-byte aligned address)
+__device__ __forceinline__ float4 ld4(const void* p, int64_t i, bool f32) {
+  if (f32) return *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i);
+  const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<const bf16_t*>(p) + i);
+  return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                     __uint_as_float(w.y & 0xffff0000u));
+}
+__device__ __forceinline__ void st4(void* p, int64_t i, bool f32, float4 v) {
+  if (f32) {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(p) + i) = v;
+  } else {
+    uint2 w;
+    w.x = pack2(v.x, v.y);
+    w.y = pack2(v.z, v.w);
+    *reinterpret_cast<uint2*>(reinterpret_cast<bf16_t*>(p) + i) = w;
+  }
+}
+__device__ __forceinline__ float4 f4(const float* p, int64_t i) { return *reinterpret_cast<const float4*>(p + i); }
+
+// One workgroup per token; 16 lanes per head, 16 heads at a time. vec: head sizes and strides that are multiples of
+// 4 with aligned bases, 4 values per lane and trip.
 __global__ void __launch_bounds__(NT) head_norm_gate_kernel(void* out, const float* o, const float* nq,
                                                            const float* abe, const void* g, int64_t gstride, bool f32,
-                                                           const float* w, int H, int dv, float eps) {
+                                                           const float* w, int H, int dv, float eps, bool vec) {
   const int64_t t = blockIdx.x;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int h = wave; h < H; h += NT / 64) {
+  const int gl = threadIdx.x & 15, grp = threadIdx.x >> 4;
+  for (int h = grp; h < H; h += NT / 16) {
     const float den = fmaxf(fabsf(nq[t * H + h]), abe[(t * H + h) * 3 + 2]) + 1e-6f;
     const float inv = 1.0f / den;
     const float* oh = o + (t * H + h) * dv;
     float ss = 0.f;
-    for (int c = lane; c < dv; c += 64) {
-      const float u = oh[c] * inv;
-      ss += u * u;
+    if (vec) {
+      for (int c = 4 * gl; c < dv; c += 64) {
+        const float4 u = f4(oh, c);
+        ss += (u.x * u.x + u.y * u.y + u.z * u.z + u.w * u.w) * inv * inv;
+      }
+    } else {
+      for (int c = gl; c < dv; c += 16) {
+        const float u = oh[c] * inv;
+        ss += u * u;
+      }
     }
-    ss = wave_sum(ss);
-    const float rsn = 1.0f / sqrtf(ss / (float)dv + eps);
-    for (int c = lane; c < dv; c += 64) {
-      const float gt = ldv(g, t * gstride + h * dv + c, f32);
-      stv(out, (t * H + h) * dv + c, f32, oh[c] * inv * rsn * w[h * dv + c] * sigmoidf(gt));
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    const float rsn = inv / sqrtf(ss / (float)dv + eps);
+    if (vec) {
+      for (int c = 4 * gl; c < dv; c += 64) {
+        const float4 u = f4(oh, c), ww = f4(w, h * dv + c), gt = ld4(g, t * gstride + h * dv + c, f32);
+        st4(out, (t * H + h) * dv + c, f32,
+            make_float4(u.x * rsn * ww.x * sigmoidf(gt.x), u.y * rsn * ww.y * sigmoidf(gt.y),
+                        u.z * rsn * ww.z * sigmoidf(gt.z), u.w * rsn * ww.w * sigmoidf(gt.w)));
+      }
+    } else {
+      for (int c = gl; c < dv; c += 16) {
+        const float gt = ldv(g, t * gstride + h * dv + c, f32);
+        stv(out, (t * H + h) * dv + c, f32, oh[c] * rsn * w[h * dv + c] * sigmoidf(gt));
+      }
     }
   }
 }
 
-// One workgroup per (token, part of the row).
+// One workgroup per (token, part of the row); the gated row is staged in LDS between its statistics and the store.
 __global__ void __launch_bounds__(NT) skip_gate_group_norm_kernel(void* out, const float* o, const void* x,
                                                                  int64_t xstride, const float* D, const void* z,
                                                                  int64_t zstride, bool f32, const float* w, int n,
-                                                                 int dv, int pw, float eps) {
-  extern __shared__ float ys[];   // [pw]
+                                                                 int dv, int pw, float eps, bool vec) {
+  extern __shared__ __attribute__((aligned(16))) float ys[];   // [pw]
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
   const int c0 = blockIdx.y * pw;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < pw; c += NT) {
-    const int col = c0 + c;
-    const float xv = ldv(x, t * xstride + col, f32), zv = ldv(z, t * zstride + col, f32);
-    const float y = (o[t * n + col] + D[col / dv] * xv) * siluf(zv);
-    ys[c] = y;
-    ss += y * y;
+  if (vec) {
+    for (int c = 4 * threadIdx.x; c < pw; c += 4 * NT) {
+      const int col = c0 + c;
+      const float4 ov = f4(o, t * n + col), xv = ld4(x, t * xstride + col, f32), zv = ld4(z, t * zstride + col, f32);
+      const float dh = D[col / dv];
+      const float4 y = make_float4((ov.x + dh * xv.x) * siluf(zv.x), (ov.y + dh * xv.y) * siluf(zv.y),
+                                   (ov.z + dh * xv.z) * siluf(zv.z), (ov.w + dh * xv.w) * siluf(zv.w));
+      *reinterpret_cast<float4*>(ys + c) = y;
+      ss += y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
+    }
+  } else {
+    for (int c = threadIdx.x; c < pw; c += NT) {
+      const int col = c0 + c;
+      const float xv = ldv(x, t * xstride + col, f32), zv = ldv(z, t * zstride + col, f32);
+      const float y = (o[t * n + col] + D[col / dv] * xv) * siluf(zv);
+      ys[c] = y;
+      ss += y * y;
+    }
   }
   ss = block_sum<NT>(ss, red);
   const float rsn = 1.0f / sqrtf(ss / (float)pw + eps);
+  if (vec) {
+    for (int c = 4 * threadIdx.x; c < pw; c += 4 * NT) {
+      const float4 y = *reinterpret_cast<const float4*>(ys + c), ww = f4(w, c0 + c);
+      st4(out, t * n + c0 + c, f32, make_float4(y.x * rsn * ww.x, y.y * rsn * ww.y, y.z * rsn * ww.z, y.w * rsn * ww.w));
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < pw; c += NT) stv(out, t * n + c0 + c, f32, ys[c] * rsn * w[c0 + c]);
 }
 
-// One workgroup per row; the averaged row is staged in LDS between its statistics and the update.
+// One workgroup per row; the averaged row is staged in LDS between its statistics and the update. bf16 rows of a
+// multiple of 8 columns: 16-byte loads and stores, 8 columns per thread and trip.
 __global__ void __launch_bounds__(NT) pair_post_norm_residual_kernel(float* resid, void* act, const void* y1,
                                                                     int64_t ys1, const float* w1, const void* y2,
                                                                     int64_t ys2, const float* w2, bool f32,
                                                                     const void* w, float mult, float eps, int W) {
-  extern __shared__ float u[];   // [W]
+  extern __shared__ __attribute__((aligned(16))) float u[];   // [W]
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
+  if (!f32 && W % 8 == 0 && ys1 % 8 == 0 && ys2 % 8 == 0 && al16(y1) && al16(y2) && al16(w) && al16(resid) &&
+      (act == nullptr || al16(act))) {
+    const uint4* p1 = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(y1) + t * ys1);
+    const uint4* p2 = reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(y2) + t * ys2);
+    float s1 = 0.f, s2 = 0.f;
+    for (int c = threadIdx.x; c < W / 8; c += NT) {
+      float a8[8], b8[8];
+      unpack8(p1[c], a8);
+      unpack8(p2[c], b8);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        s1 += a8[q] * a8[q];
+        s2 += b8[q] * b8[q];
+      }
+    }
+    s1 = block_sum<NT>(s1, red);
+    s2 = block_sum<NT>(s2, red);
+    const float r1 = 0.5f / sqrtf(s1 / (float)W + eps), r2 = 0.5f / sqrtf(s2 / (float)W + eps);
+    float su = 0.f;
+    for (int c = threadIdx.x; c < W / 8; c += NT) {
+      float a8[8], b8[8];
+      unpack8(p1[c], a8);
+      unpack8(p2[c], b8);
+      const float4 wa0 = f4(w1, 8 * c), wa1 = f4(w1, 8 * c + 4), wb0 = f4(w2, 8 * c), wb1 = f4(w2, 8 * c + 4);
+      const float wa[8] = {wa0.x, wa0.y, wa0.z, wa0.w, wa1.x, wa1.y, wa1.z, wa1.w};
+      const float wb[8] = {wb0.x, wb0.y, wb0.z, wb0.w, wb1.x, wb1.y, wb1.z, wb1.w};
+      float v[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        v[q] = a8[q] * r1 * wa[q] + b8[q] * r2 * wb[q];
+        su += v[q] * v[q];
+      }
+      *reinterpret_cast<float4*>(u + 8 * c) = make_float4(v[0], v[1], v[2], v[3]);
+      *reinterpret_cast<float4*>(u + 8 * c + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+    su = block_sum<NT>(su, red);
+    const float ru = mult / sqrtf(su / (float)W + eps);
+    float4* rr = reinterpret_cast<float4*>(resid + t * W);
+    for (int c = threadIdx.x; c < W / 8; c += NT) {
+      float g8[8];
+      unpack8(reinterpret_cast<const uint4*>(w)[c], g8);
+      const float4 u0 = *reinterpret_cast<const float4*>(u + 8 * c), u1 = *reinterpret_cast<const float4*>(u + 8 * c + 4);
+      const float uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+      const float4 a0 = rr[2 * c], a1 = rr[2 * c + 1];
+      float o8[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+      for (int q = 0; q < 8; ++q) o8[q] += uv[q] * ru * (1.0f + g8[q]);
+      rr[2 * c] = make_float4(o8[0], o8[1], o8[2], o8[3]);
+      rr[2 * c + 1] = make_float4(o8[4], o8[5], o8[6], o8[7]);
+      if (act) reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(act) + t * W)[c] = pack8(o8);
+    }
+    return;
+  }
   float s1 = 0.f, s2 = 0.f;
   for (int c = threadIdx.x; c < W; c += NT) {
     const float a = ldv(y1, t * ys1 + c, f32), b = ldv(y2, t * ys2 + c, f32);
@@ -587,7 +707,11 @@ hipError_t launch_head_norm_gate(void* out, const float* o, const float* nq, con
                                  hipStream_t s) {
   if (T == 0) return hipSuccess;
   if (H < 1 || vdim < 1) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(head_norm_gate_kernel, dim3(T), dim3(NT), 0, s, out, o, nq, abe, g, gstride, f32, w, H, vdim, eps);
+  const bool vec = vdim % 4 == 0 && gstride % 4 == 0 && (reinterpret_cast<uintptr_t>(g) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(o) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  hipLaunchKernelGGL(head_norm_gate_kernel, dim3(T), dim3(NT), 0, s, out, o, nq, abe, g, gstride, f32, w, H, vdim, eps,
+                     vec);
   return hipGetLastError();
 }
 
@@ -597,8 +721,11 @@ hipError_t launch_skip_gate_group_norm(void* out, const float* o, const void* x,
   if (T == 0) return hipSuccess;
   const int n = H * vdim;
   if (H < 1 || vdim < 1 || parts < 1 || parts > 65535 || n % parts || n / parts > 16384) return hipErrorInvalidValue;
+  auto a16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool vec = vdim % 4 == 0 && (n / parts) % 4 == 0 && xstride % 4 == 0 && zstride % 4 == 0 && a16(o) && a16(x) &&
+                   a16(z) && a16(w) && a16(out);
   hipLaunchKernelGGL(skip_gate_group_norm_kernel, dim3(T, parts), dim3(NT), (size_t)(n / parts) * sizeof(float), s,
-                     out, o, x, xstride, D, z, zstride, f32, w, n, vdim, n / parts, eps);
+                     out, o, x, xstride, D, z, zstride, f32, w, n, vdim, n / parts, eps, vec);
   return hipGetLastError();
 }
 

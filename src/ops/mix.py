@@ -264,6 +264,34 @@ def moe_output_weighted(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w:
 
     if e == 0:
         return finish(torch.empty(0, h, dtype=x.dtype, device=x.device), None)
+    buckets = max(e, int(n_route))
+    if x.dtype == torch.bfloat16 and t <= 128:
+        # decode-sized steps: the framework's expert-streaming grouped GEMM (every routed expert's weights streamed
+        # once; rows gathered in expert-sorted order by the kernel; no host read, hipGraph-capturable). Identity
+        # entries sort behind the last real expert and run nothing.
+        from src import ops
+
+        tiles = None
+        if ops.native_available() and h % 32 == 0 and w2.shape[2] % 32 == 0:
+            try:
+                b = ops._bucket(t)
+                tiles = (ops._generic_tile(w13.shape[1], h, 0, b, max_sk=1)[:2],
+                         ops._generic_tile(h, w2.shape[2], 0, b, max_sk=1)[:2])
+            except ValueError:
+                tiles = None
+        if tiles is not None:
+            ck = ops._kern()
+            (wr1, kc1), (wr2, kc2) = tiles
+            offsets = torch.empty(buckets + 1, dtype=torch.int32, device=x.device)
+            sorted_idx = torch.empty(n, dtype=torch.int32, device=x.device)
+            pos = torch.empty(n, dtype=torch.int32, device=x.device)
+            kern.moe_align(offsets, sorted_idx, pos, ids.reshape(-1).contiguous(), buckets)
+            g = torch.empty(n, w13.shape[1], dtype=x.dtype, device=x.device)
+            ys = torch.empty(n, h, dtype=x.dtype, device=x.device)
+            ck.gemm_decode_grouped(g, x, w13, offsets, 0, wr1, kc1, sorted_idx, k, t, 1)
+            ck.gemm_decode_grouped(ys, gated_act(g, kind, limit, alpha), w2, offsets, 0, wr2, kc2,
+                                   ops._NO_ROWS(x.device), 1, t, 1)
+            return finish(ys, pos)
     if n <= MOE_BMM_MAX_ROWS or torch.cuda.is_current_stream_capturing():
         # decode-sized steps: the routed experts' weights gathered per row for two batched products (no host read,
         # hipGraph-capturable); an identity entry runs expert E - 1 and its product is ignored by the sum
@@ -274,7 +302,6 @@ def moe_output_weighted(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, w:
         return finish(ys, None)
     # prompt-sized steps: rows sorted by expert (identity entries sort last and run nothing), one library GEMM pair
     # per real expert over its rows
-    buckets = max(e, int(n_route))
     offsets = torch.empty(buckets + 1, dtype=torch.int32, device=x.device)
     sorted_idx = torch.empty(n, dtype=torch.int32, device=x.device)
     pos = torch.empty(n, dtype=torch.int32, device=x.device)
