@@ -9,8 +9,9 @@
 //   selective_scan            S[c, :] <- exp(d A[c, :]) S[c, :] + d x B; y = S[c, :] . C + D x; y * silu(z): a
 //                             channel's states in the registers of 1 - 4 lanes for the whole step
 //   exp_gate_scan             log-space input / forget gates under a running maximum: a wave-wide scan over tokens
-//   gated_linear_attn         S <- a S + b k v^T, o = S^T q (+ normaliser n <- a n + b k, n . q): one workgroup per
-//                             (sequence, head, block of columns), the state in registers (a column per lane quad)
+//   gated_linear_attn         S <- a S + b k v^T, o = S^T q: one workgroup per (sequence, head, block of columns), the
+//                             state in registers (a column per lane quad); the normaliser n <- a n + b k with its
+//                             read-out n . q rides on the first wave
 //   head_norm_gate            o / (max(|n . q|, floor) + 1e-6), per-head RMS norm, weight, sigmoid gate
 //   skip_gate_group_norm      (o + D x) * silu(z), RMS norm in equal parts of the row, weight
 //   pair_post_norm_residual   resid += mult * rms((rms(y1) w1 + rms(y2) w2) / 2) * (1 + w)
@@ -31,6 +32,14 @@ __device__ __forceinline__ void stv(void* p, int64_t i, bool f32, float v) {
     reinterpret_cast<float*>(p)[i] = v;
   else
     reinterpret_cast<bf16_t*>(p)[i] = f2bf(v);
+}
+// the same with the storage type known at compile time: no branch around the load, so a run of loads stays in flight
+// together (behind a run-time branch each load is waited for before the next one issues)
+template <bool F32> __device__ __forceinline__ float ldt(const void* p, int64_t i) {
+  if constexpr (F32)
+    return reinterpret_cast<const float*>(p)[i];
+  else
+    return bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
 }
 // the value as the activation dtype would hold it
 __device__ __forceinline__ float rnd(float v, bool f32) { return f32 ? v : bf2f(f2bf(v)); }
@@ -201,11 +210,24 @@ __global__ void __launch_bounds__(NT) conv_tail_update_kernel(float* conv_state,
 constexpr int TB = 16;   // tokens staged per trip
 constexpr int SCH = 256; // threads per workgroup of the scan
 
-// One workgroup per (block of channels, sequence). A channel's N states are split over LPC lanes (NP each) and stay
-// in registers for the whole step; a token costs a lane NP exponentials and 3 NP multiply-adds, plus a reduction
-// over the LPC lanes. B_t and C_t come from LDS as float4 broadcasts; x, step size and z of TB tokens are staged
-// per trip.
-// exp(d * A): fp32 steps use expf; bf16 steps fold log2(e) into A once and use the hardware's 2^x (v_exp_f32)
+// softplus in bf16 steps: hardware exponential and logarithm (v_exp_f32 / v_log_f32), a series where 1 + e^z rounds
+template <bool FAST> __device__ __forceinline__ float step_size(float z) {
+  if constexpr (FAST) {
+    const float e = __expf(-fabsf(z));
+    const float l = e < 9.765625e-4f ? e - 0.5f * e * e : __logf(1.0f + e);
+    return fmaxf(z, 0.f) + l;
+  } else {
+    return softplusf(z);
+  }
+}
+// silu(z): bf16 steps use the hardware's exponential and reciprocal
+template <bool FAST> __device__ __forceinline__ float gate_of(float z) {
+  if constexpr (FAST)
+    return z * __builtin_amdgcn_rcpf(1.0f + __expf(-z));
+  else
+    return siluf(z);
+}
+// exp(d * A): fp32 steps use expf; bf16 steps fold log2(e) into A once and use the hardware's 2^x
 template <bool FAST> __device__ __forceinline__ float decay_of(float d, float a) {
   if constexpr (FAST)
     return __builtin_amdgcn_exp2f(d * a);
@@ -213,18 +235,19 @@ template <bool FAST> __device__ __forceinline__ float decay_of(float d, float a)
     return expf(d * a);
 }
 
+// One workgroup per (block of channels, sequence). A channel's N states are split over LPC lanes (NP each) and stay
+// in registers for the whole step; a token costs a lane NP exponentials and 3 NP multiply-adds, plus a reduction
+// over the LPC lanes. B_t and C_t of TB tokens are staged in LDS per trip and read as float4 broadcasts; every lane
+// loads its channel's x, step size and z of the trip into registers up front, so their latencies overlap.
 template <int NP, int LPC, bool FAST>
 __global__ void __launch_bounds__(SCH) selective_scan_kernel(SelectiveScanArgs a, RaggedRows r) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   constexpr int NPAD = NP * LPC, CH = SCH / LPC;
   float* Bs = sm;                     // [TB][NPAD], zero beyond N
   float* Cs = Bs + TB * NPAD;         // [TB][NPAD]
-  float* xs = Cs + TB * NPAD;         // [TB][CH]
-  float* ds = xs + TB * CH;           // [TB][CH]
-  float* zs = ds + TB * CH;           // [TB][CH]
   const int s = blockIdx.y, tid = threadIdx.x;
   const int cl = tid / LPC, part = tid % LPC;
-  const int c0 = blockIdx.x * CH, c = c0 + cl;
+  const int c = blockIdx.x * CH + cl;
   const int I = a.I, N = a.N;
   const bool f32 = a.f32;
   const int q0 = r.cu_q ? r.cu_q[s] : s;
@@ -232,71 +255,99 @@ __global__ void __launch_bounds__(SCH) selective_scan_kernel(SelectiveScanArgs a
   if (L <= 0) return;
   const bool fresh = r.positions[q0] <= 0;
   const bool live = c < I;
-  float* st = a.state + ((int64_t)r.state_slots[s] * I + (live ? c : 0)) * N;
+  const int cc = live ? c : 0;
+  float* st = a.state + ((int64_t)r.state_slots[s] * I + cc) * N;
+  const float* Ap = a.A + (int64_t)cc * N;
   float S[NP], A[NP];
+  constexpr float LOG2E = 1.4426950408889634f;
+  if (N % 4 == 0) {
 #pragma unroll
-  for (int i = 0; i < NP; ++i) {
-    const int n = part * NP + i;
-    const bool ok = live && n < N;
-    S[i] = (ok && !fresh) ? st[n] : 0.f;
-    A[i] = ok ? a.A[(int64_t)c * N + n] * (FAST ? 1.4426950408889634f : 1.0f) : 0.f;
+    for (int i = 0; i < NP / 4; ++i) {
+      const int n = part * NP + 4 * i;
+      const bool ok = live && n < N;
+      const float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      const float4 sv = (ok && !fresh) ? *reinterpret_cast<const float4*>(st + n) : z4;
+      const float4 av = ok ? *reinterpret_cast<const float4*>(Ap + n) : z4;
+      S[4 * i] = sv.x, S[4 * i + 1] = sv.y, S[4 * i + 2] = sv.z, S[4 * i + 3] = sv.w;
+      A[4 * i] = av.x, A[4 * i + 1] = av.y, A[4 * i + 2] = av.z, A[4 * i + 3] = av.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int n = part * NP + i;
+      const bool ok = live && n < N;
+      S[i] = (ok && !fresh) ? st[n] : 0.f;
+      A[i] = ok ? Ap[n] : 0.f;
+    }
   }
-  const float Dc = live ? a.D[c] : 0.f;
+  if (FAST) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) A[i] *= LOG2E;
+  }
+  const float Dc = a.D[cc], dtb = a.dt_bias[cc];
   for (int t0 = 0; t0 < L; t0 += TB) {
     const int nb = min(TB, L - t0);
     __syncthreads();
     for (int e = tid; e < nb * NPAD; e += SCH) {
       const int tt = e / NPAD, n = e % NPAD;
       const int64_t base = (int64_t)(q0 + t0 + tt) * a.bcstride;
-      Bs[e] = n < N ? ldv(a.bc, base + a.boff + n, f32) : 0.f;
-      Cs[e] = n < N ? ldv(a.bc, base + a.coff + n, f32) : 0.f;
+      Bs[e] = n < N ? ldt<!FAST>(a.bc, base + a.boff + n) : 0.f;
+      Cs[e] = n < N ? ldt<!FAST>(a.bc, base + a.coff + n) : 0.f;
     }
-    for (int e = tid; e < nb * CH; e += SCH) {
-      const int tt = e / CH, cc = c0 + e % CH;
-      const int64_t row = q0 + t0 + tt;
-      const bool ok = cc < I;
-      xs[e] = ok ? ldv(a.x, row * a.xstride + cc, f32) : 0.f;
-      ds[e] = ok ? softplusf(ldv(a.dt, row * a.dtstride + cc, f32) + a.dt_bias[cc]) : 0.f;
-      zs[e] = ok ? ldv(a.z, row * a.zstride + cc, f32) : 0.f;
+    float xr[TB], dr[TB], zr[TB];
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) {
+      const int64_t row = q0 + t0 + (tt < nb ? tt : 0);
+      xr[tt] = ldt<!FAST>(a.x, row * a.xstride + cc);
+      dr[tt] = ldt<!FAST>(a.dt, row * a.dtstride + cc);
+      zr[tt] = ldt<!FAST>(a.z, row * a.zstride + cc);
     }
     __syncthreads();
-    for (int tt = 0; tt < nb; ++tt) {
-      const float x = xs[tt * CH + cl], d = ds[tt * CH + cl];
-      const float dx = d * x;
-      const float4* Bt = reinterpret_cast<const float4*>(Bs + tt * NPAD + part * NP);
-      const float4* Ct = reinterpret_cast<const float4*>(Cs + tt * NPAD + part * NP);
-      float y0 = 0.f, y1 = 0.f;
 #pragma unroll
-      for (int i = 0; i < NP / 4; ++i) {
-        const float4 b4 = Bt[i], c4 = Ct[i];
-        S[4 * i] = decay_of<FAST>(d, A[4 * i]) * S[4 * i] + dx * b4.x;
-        S[4 * i + 1] = decay_of<FAST>(d, A[4 * i + 1]) * S[4 * i + 1] + dx * b4.y;
-        S[4 * i + 2] = decay_of<FAST>(d, A[4 * i + 2]) * S[4 * i + 2] + dx * b4.z;
-        S[4 * i + 3] = decay_of<FAST>(d, A[4 * i + 3]) * S[4 * i + 3] + dx * b4.w;
-        y0 += S[4 * i] * c4.x + S[4 * i + 2] * c4.z;
-        y1 += S[4 * i + 1] * c4.y + S[4 * i + 3] * c4.w;
-      }
-      float y = y0 + y1;
-      if (LPC > 1) y += __shfl_xor(y, 1, 64);
-      if (LPC > 2) y += __shfl_xor(y, 2, 64);
-      if (part == 0 && live) {
-        const float z = zs[tt * CH + cl];
-        stv(a.out, (int64_t)(q0 + t0 + tt) * I + c, f32, (y + Dc * x) * siluf(z));
+    for (int tt = 0; tt < TB; ++tt) {
+      if (tt < nb) {
+        const float x = xr[tt], d = step_size<FAST>(dr[tt] + dtb);
+        const float dx = d * x;
+        const float4* Bt = reinterpret_cast<const float4*>(Bs + tt * NPAD + part * NP);
+        const float4* Ct = reinterpret_cast<const float4*>(Cs + tt * NPAD + part * NP);
+        float y0 = 0.f, y1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NP / 4; ++i) {
+          const float4 b4 = Bt[i], c4 = Ct[i];
+          S[4 * i] = decay_of<FAST>(d, A[4 * i]) * S[4 * i] + dx * b4.x;
+          S[4 * i + 1] = decay_of<FAST>(d, A[4 * i + 1]) * S[4 * i + 1] + dx * b4.y;
+          S[4 * i + 2] = decay_of<FAST>(d, A[4 * i + 2]) * S[4 * i + 2] + dx * b4.z;
+          S[4 * i + 3] = decay_of<FAST>(d, A[4 * i + 3]) * S[4 * i + 3] + dx * b4.w;
+          y0 += S[4 * i] * c4.x + S[4 * i + 2] * c4.z;
+          y1 += S[4 * i + 1] * c4.y + S[4 * i + 3] * c4.w;
+        }
+        float y = y0 + y1;
+        if (LPC > 1) y += __shfl_xor(y, 1, 64);
+        if (LPC > 2) y += __shfl_xor(y, 2, 64);
+        if (part == 0 && live) stv(a.out, (int64_t)(q0 + t0 + tt) * I + c, f32, (y + Dc * x) * gate_of<FAST>(zr[tt]));
       }
     }
   }
   if (live) {
+    if (N % 4 == 0) {
 #pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      const int n = part * NP + i;
-      if (n < N) st[n] = S[i];
+      for (int i = 0; i < NP / 4; ++i) {
+        const int n = part * NP + 4 * i;
+        if (n < N) *reinterpret_cast<float4*>(st + n) = make_float4(S[4 * i], S[4 * i + 1], S[4 * i + 2], S[4 * i + 3]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const int n = part * NP + i;
+        if (n < N) st[n] = S[i];
+      }
     }
   }
 }
 
 template <int NP, int LPC> hipError_t launch_scan_one(const SelectiveScanArgs& a, RaggedRows r, hipStream_t s) {
   constexpr int CH = SCH / LPC;
-  const size_t smem = (size_t)TB * (2 * NP * LPC + 3 * CH) * sizeof(float);
+  const size_t smem = (size_t)TB * 2 * NP * LPC * sizeof(float);
   const dim3 grid((a.I + CH - 1) / CH, r.num_seqs);
   if (a.f32)
     hipLaunchKernelGGL((selective_scan_kernel<NP, LPC, false>), grid, dim3(SCH), smem, s, a, r);
@@ -352,11 +403,13 @@ __global__ void __launch_bounds__(64) exp_gate_scan_kernel(float* abe, const voi
 
 // ---------------------------------------------------------------------------------------- matrix recurrence
 // One workgroup per (head, sequence, block of VC columns). The state lives in registers for the whole step: column j
-// is split over the 4 lanes of a quad, lane `part` holding rows [part * DP, (part + 1) * DP). With a normaliser, column
-// block 0 carries it as one more column (the quad after the last value column) whose value is 1. A token costs each
-// lane 2 * DP multiply-adds and one quad reduction; q (scaled) and k come from LDS as float4 broadcasts, b scales the
-// value.
-template <int DP>
+// is split over the 4 lanes of a quad, lane `part` holding rows [part * DP, (part + 1) * DP). A token costs each lane
+// 2 * DP multiply-adds and one quad reduction; q (scaled) and k come from LDS as float4 broadcasts, b scales the
+// value. The normaliser n <- a n + b k (a vector of `dim` rows, RP per lane) is carried by the first wave of column
+// block 0, which runs a trip's tokens over the staged k and q once more after its columns and reduces the TB dot
+// products n . q over its lanes. (As a column of its own the normaliser would add a ninth wave to workgroups of 512
+// threads; measured, that ran 1.8x slower than the kernel without it, and a one-wave launch beside it 1.7x.)
+template <int DP, bool F32>
 __global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs a, RaggedRows r, int VC) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   constexpr int DPAD = 4 * DP;
@@ -369,36 +422,36 @@ __global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs
   const int v0 = blockIdx.z * VC;
   const int ncol = min(VC, dv - v0);
   const int j = tid >> 2, part = tid & 3;
-  const bool is_n = a.n_state != nullptr && blockIdx.z == 0 && j == ncol;   // this quad holds the normaliser
-  const bool used = j < ncol || is_n;
   const int g = h / (H / a.groups);
   const int q0 = r.cu_q ? r.cu_q[s] : s;
   const int L = r.cu_q ? r.cu_q[s + 1] - q0 : 1;
   if (L <= 0) return;
   const bool fresh = r.positions[q0] <= 0;
-  const bool f32 = a.f32;
-  const int64_t slot = r.state_slots[s];
-  // column j's rows: stride dv in the matrix state, 1 in the normaliser
-  float* st = is_n ? a.n_state + (slot * H + h) * d : a.state + (slot * H + h) * (int64_t)d * dv + v0 + j;
-  const int64_t rs = is_n ? 1 : dv;
+  float* st = a.state + ((int64_t)r.state_slots[s] * H + h) * (int64_t)d * dv + v0 + j;
   float S[DP];
 #pragma unroll
   for (int i = 0; i < DP; ++i) {
     const int row = part * DP + i;
-    S[i] = (!fresh && row < d && used) ? st[(int64_t)row * rs] : 0.f;
+    S[i] = (!fresh && row < d && j < ncol) ? st[(int64_t)row * dv] : 0.f;
   }
+  constexpr int RP = DPAD > 64 ? DPAD / 64 : 1;
+  const bool norm = a.n_state != nullptr && blockIdx.z == 0 && tid < 64;   // wave-uniform
+  float* nst = norm ? a.n_state + ((int64_t)r.state_slots[s] * H + h) * d : nullptr;
+  float nv[RP];
+#pragma unroll
+  for (int i = 0; i < RP; ++i) nv[i] = (norm && !fresh && tid + 64 * i < d) ? nst[tid + 64 * i] : 0.f;
   for (int t0 = 0; t0 < L; t0 += TB) {
     const int nb = min(TB, L - t0);
     __syncthreads();
     for (int e = tid; e < nb * DPAD; e += nthr) {
       const int tt = e / DPAD, c = e % DPAD;
       const int64_t base = (int64_t)(q0 + t0 + tt) * a.xstride + g * d + c;
-      qs[e] = c < d ? ldv(a.x, base + a.qoff, f32) * a.qscale : 0.f;
-      ks[e] = c < d ? ldv(a.x, base + a.koff, f32) : 0.f;
+      qs[e] = c < d ? ldt<F32>(a.x, base + a.qoff) * a.qscale : 0.f;
+      ks[e] = c < d ? ldt<F32>(a.x, base + a.koff) : 0.f;
     }
     for (int e = tid; e < nb * VC; e += nthr) {
       const int tt = e / VC, c = e % VC;
-      vs[e] = c < ncol ? ldv(a.x, (int64_t)(q0 + t0 + tt) * a.xstride + a.voff + h * dv + v0 + c, f32) : 0.f;
+      vs[e] = c < ncol ? ldt<F32>(a.x, (int64_t)(q0 + t0 + tt) * a.xstride + a.voff + h * dv + v0 + c) : 0.f;
     }
     for (int e = tid; e < 2 * nb; e += nthr) as[e] = a.ab[((int64_t)(q0 + t0 + (e >> 1)) * H + h) * a.abw + (e & 1)];
     __syncthreads();
@@ -406,7 +459,7 @@ __global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs
       const float4* kt = reinterpret_cast<const float4*>(ks + tt * DPAD + part * DP);
       const float4* qt = reinterpret_cast<const float4*>(qs + tt * DPAD + part * DP);
       const float2 ab = *reinterpret_cast<const float2*>(as + 2 * tt);
-      const float vj = (is_n ? 1.0f : (j < ncol ? vs[tt * VC + j] : 0.f)) * ab.y;
+      const float vj = (j < ncol ? vs[tt * VC + j] : 0.f) * ab.y;
       const float dec = ab.x;
       float o0 = 0.f, o1 = 0.f;
 #pragma unroll
@@ -422,31 +475,60 @@ __global__ void __launch_bounds__(1024) gated_linear_attn_kernel(GatedLinearArgs
       float o = o0 + o1;
       o += __shfl_xor(o, 1, 64);
       o += __shfl_xor(o, 2, 64);
-      if (part == 0 && used) {
-        const int64_t row = q0 + t0 + tt;
-        if (is_n)
-          a.nq[row * H + h] = o;
-        else
-          a.out[(row * H + h) * dv + v0 + j] = o;
+      if (part == 0 && j < ncol) a.out[((int64_t)(q0 + t0 + tt) * H + h) * dv + v0 + j] = o;
+    }
+    if (norm) {
+      float p[TB];
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt) {
+        float acc = 0.f;
+        if (tt < nb) {
+          const float2 ab = *reinterpret_cast<const float2*>(as + 2 * tt);
+#pragma unroll
+          for (int i = 0; i < RP; ++i) {
+            const int row = tid + 64 * i;
+            if (row < DPAD) {
+              nv[i] = nv[i] * ab.x + ab.y * ks[tt * DPAD + row];
+              acc += nv[i] * qs[tt * DPAD + row];
+            }
+          }
+        }
+        p[tt] = xor32_sum(acc);
+      }
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt) {
+        float v = p[tt];
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        if (tid == 0 && tt < nb) a.nq[(int64_t)(q0 + t0 + tt) * H + h] = v;
       }
     }
   }
-  if (used) {
+  if (j < ncol) {
 #pragma unroll
     for (int i = 0; i < DP; ++i) {
       const int row = part * DP + i;
-      if (row < d) st[(int64_t)row * rs] = S[i];
+      if (row < d) st[(int64_t)row * dv] = S[i];
     }
+  }
+  if (norm) {
+#pragma unroll
+    for (int i = 0; i < RP; ++i)
+      if (tid + 64 * i < d) nst[tid + 64 * i] = nv[i];
   }
 }
 
-template <int DP> hipError_t launch_gla_dp(const GatedLinearArgs& a, RaggedRows r, hipStream_t s) {
+template <int DP, bool F32> hipError_t launch_gla_dp(const GatedLinearArgs& a, RaggedRows r, hipStream_t s) {
   const int VC = a.vdim < 128 ? a.vdim : 128;
   const int nvc = (a.vdim + VC - 1) / VC;
-  const int threads = (4 * (VC + (a.n_state ? 1 : 0)) + 63) / 64 * 64;
+  const int threads = (4 * VC + 63) / 64 * 64;
   const size_t smem = (size_t)(2 * TB * 4 * DP + TB * VC + 2 * TB) * sizeof(float);
-  hipLaunchKernelGGL(gated_linear_attn_kernel<DP>, dim3(a.heads, r.num_seqs, nvc), dim3(threads), smem, s, a, r, VC);
+  hipLaunchKernelGGL((gated_linear_attn_kernel<DP, F32>), dim3(a.heads, r.num_seqs, nvc), dim3(threads), smem, s, a, r,
+                     VC);
   return hipGetLastError();
+}
+template <int DP> hipError_t launch_gla_dp(const GatedLinearArgs& a, RaggedRows r, hipStream_t s) {
+  return a.f32 ? launch_gla_dp<DP, true>(a, r, s) : launch_gla_dp<DP, false>(a, r, s);
 }
 
 // ------------------------------------------------------------------------------------------------ epilogues
