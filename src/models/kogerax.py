@@ -620,7 +620,7 @@ class KogeraxLM:
                 else:
                     # the shared expert's gate row rides below the router's rows: one product gives both
                     lw.router = rnd(f.n_route + (1 if f.shared_ff else 0), h, scale=init_std * 4)
-                    lw.correction = rnd(f.n_route, scale=0.02, dt=torch.float32)
+                    lw.correction = torch.zeros(f.n_route, dtype=torch.float32, device=self.device)
                     lw.w13 = rnd(f.experts, 2 * f.expert_ff, h)
                     lw.w2 = rnd(f.experts, h, f.expert_ff)
                     if f.shared_ff:
