@@ -79,7 +79,7 @@ def kogerax_arch(z):
                        rot_scaling=(8.0, 1.0, 4.0, 8192.0), qk_norm=True, head_norm=True, norm_after_rot=True,
                        norm_weights=False, has_sink=False)
     scan = SelectiveScanSpec(inner=z["s_inner"], state=z["s_state"], dt_rank=z["s_rank"], conv=z["conv"])
-    lstm = MLstmSpec(heads=z["l_heads"], dim=z["l_dim"], vdim=z["l_vdim"], gate_cap=15.0)
+    lstm = MLstmSpec(heads=z["l_heads"], dim=z["l_dim"], vdim=z["l_vdim"], gate_cap=12.0)
     ssd = Mamba2Spec(heads=z["m_heads"], vdim=z["m_vdim"], state=z["m_state"], groups=z["m_groups"], conv=z["conv"],
                      norm_groups=1)
     dense = GatedMlpSpec("dense", ff=z["ff"])
@@ -152,7 +152,7 @@ def kernels(z, a, size):
     ib, fb = torch.zeros(H, device=dev), torch.full((H,), 2.0, device=dev)
     for mode, T2, rag in rags:
         x = torch.randn(T2, 2 * H, device=dev).to(bf)
-        t = _time(lambda: rec.exp_gate_scan(x, 0, H, ib, fb, 15.0, mst, H, rag), a.iters)
+        t = _time(lambda: rec.exp_gate_scan(x, 0, H, ib, fb, 12.0, mst, H, rag), a.iters)
         emit({"design": "kogerax", "kernel": "exp_gate_scan", "mode": mode, "ms": round(t * 1e3, 4)})
     # ---- selective scan
     I, N, R = z["s_inner"], z["s_state"], z["s_rank"]
