@@ -349,7 +349,7 @@ __global__ void __launch_bounds__(NT) combine_weighted_kernel(float* out, float*
                                                              const int* ids, int E, const void* extra,
                                                              const float* gate, int K, int H, const void* w, bool w_f32,
                                                              bool unit, float eps, float mult) {
-  extern __shared__ float acc[];   // [H]
+  extern __shared__ __attribute__((aligned(16))) float acc[];   // [H]
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
   const float gt = extra ? (gate ? gate[t] : 1.0f) : 0.f;
@@ -374,10 +374,9 @@ __global__ void __launch_bounds__(NT) combine_weighted_kernel(float* out, float*
         for (int q = 0; q < 8; ++q) a[q] += wt * v[q];
       }
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        acc[8 * c + q] = a[q];
-        ss += a[q] * a[q];
-      }
+      for (int q = 0; q < 8; ++q) ss += a[q] * a[q];
+      *reinterpret_cast<float4*>(acc + 8 * c) = make_float4(a[0], a[1], a[2], a[3]);
+      *reinterpret_cast<float4*>(acc + 8 * c + 4) = make_float4(a[4], a[5], a[6], a[7]);
     }
   } else {
     for (int c = threadIdx.x; c < H; c += NT) {
@@ -398,6 +397,23 @@ __global__ void __launch_bounds__(NT) combine_weighted_kernel(float* out, float*
   if (resid == nullptr) return;
   ss = block_sum<NT>(ss, red);
   const float rs = mult / sqrtf(ss / (float)H + eps);
+  if (vec && !w_f32 && aligned16(w) && aligned16(resid) && (act == nullptr || aligned16(act))) {
+    float4* rr = reinterpret_cast<float4*>(resid + t * H);
+    for (int c = threadIdx.x; c < H / 8; c += NT) {
+      float g[8];
+      unpack8(reinterpret_cast<const uint4*>(w)[c], g);
+      const float4 u0 = *reinterpret_cast<const float4*>(acc + 8 * c), u1 = *reinterpret_cast<const float4*>(acc + 8 * c + 4);
+      const float u[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+      const float4 r0 = rr[2 * c], r1 = rr[2 * c + 1];
+      float o[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+      for (int q = 0; q < 8; ++q) o[q] += u[q] * rs * (unit ? g[q] + 1.0f : g[q]);
+      rr[2 * c] = make_float4(o[0], o[1], o[2], o[3]);
+      rr[2 * c + 1] = make_float4(o[4], o[5], o[6], o[7]);
+      if (act) reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(act) + t * H)[c] = pack8(o);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < H; c += NT) {
     float g = ldv(w, c, w_f32);
     if (unit) g += 1.0f;
