@@ -3,9 +3,11 @@ Dtype-generic ops (bf16 or fp32 storage, fp32 arithmetic) on the ``src/_Cmix`` H
 
 * :func:`rms_norm_ext`, :func:`post_norm_residual` — RMS norms with a plain weight or a `1 + w` gain,
   the second one applied to a sublayer's OUTPUT and added into an fp32 residual stream;
-* :func:`gated_act` — SiLU-gated and clamped sigmoid-gated feed-forward activations;
+* :func:`gated_act` — SiLU-gated, clamped sigmoid-gated and GELU-gated feed-forward activations;
 * :func:`route_sigmoid_topk`, :func:`moe_input_scaled` — sigmoid-scored top-k routing whose weight scales
   the expert's input, with an optional always-on shared expert;
+* :func:`route_softmax_topk`, :func:`moe_output_weighted` — softmax-scored top-k routing with a correction that
+  enters the choice only, identity experts, renormalised weights on the experts' outputs and a gated shared expert;
 * :func:`latent_kv_write`, :func:`latent_attn` — latent (compressed-KV) attention over a paged cache of
   [latent | rotated shared key] rows, with a sliding window and a per-head softmax sink.
 
